@@ -1,0 +1,72 @@
+"""ctypes binding of libdistca_ca.so (the C ABI declared in include/distca_ca.h).
+
+The library is the product: there is no Python or CPU fallback.  Importing this module
+without a built library raises, and every wrapper turns a non-zero return code into a
+RuntimeError carrying distca_last_error().
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdistca_ca.so")
+
+ABI_VERSION = 1
+
+
+class CaParams(Structure):
+    """struct distca_ca_params (include/distca_ca.h)."""
+    _fields_ = [
+        ("num_tasks", c_int32), ("total_q", c_int32), ("total_k", c_int32),
+        ("num_heads_q", c_int32), ("num_heads_kv", c_int32), ("head_dim", c_int32),
+        ("max_seqlen_q", c_int32), ("max_seqlen_k", c_int32),
+        ("softmax_scale", c_float), ("causal", c_int32), ("deterministic", c_int32),
+        ("reserved", c_int32),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/distca_ca.h declares
+SYMBOLS = {
+    "distca_last_error": (c_char_p, []),
+    "distca_abi_version": (c_int, []),
+    "distca_memcpy_non_cp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "distca_memcpy_cp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p]),
+    "distca_grad_sum": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "distca_ca_fwd_workspace_bytes": (c_int64, [POINTER(CaParams)]),
+    "distca_ca_bwd_workspace_bytes": (c_int64, [POINTER(CaParams)]),
+    "distca_ca_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                              POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_schedule_host": (c_int64, [c_int, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64]),
+    "distca_ca_tile_shape": (c_int, [c_int, POINTER(CaParams), POINTER(c_int32 * 2)]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the library once; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m distca_amd._build` (needs hipcc); "
+            "distca_amd has no fallback path")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    if lib.distca_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"libdistca_ca.so ABI {lib.distca_abi_version()} != binding ABI {ABI_VERSION}: rebuild")
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().distca_last_error()
+        raise RuntimeError(f"{what} failed ({rc}): {msg.decode() if msg else ''}")

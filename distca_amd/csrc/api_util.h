@@ -1,0 +1,33 @@
+// Host-side helpers shared by the C-ABI entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/distca_ca.h"
+
+namespace distca {
+
+char *error_buffer();  // thread-local, 512 bytes
+
+inline int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return DISTCA_OK;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Number of compute units of the current device (cached per device id).
+int num_compute_units();
+
+}  // namespace distca

@@ -1,0 +1,84 @@
+// Tile geometry of the attention kernels and the checks every entry point shares.
+#pragma once
+#include <math.h>
+#include <stdlib.h>
+
+#include "api_util.h"
+#include "sched.h"
+
+namespace distca {
+
+constexpr int kHeadDim = 128;
+constexpr int kWaves = 4;  // waves per workgroup in every attention kernel
+
+// Forward: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles of 64 keys.
+#ifndef DISTCA_FWD_MSUB
+#define DISTCA_FWD_MSUB 2
+#endif
+constexpr int kFwdMsub = DISTCA_FWD_MSUB;
+constexpr int kFwdRows = kWaves * 32 * kFwdMsub;
+constexpr int kFwdKV = 64;
+
+// Backward: each wave owns BWD_KSUB sub-tiles of 32 keys; query rows are streamed in blocks
+// of 32 * BWD_MSUB flattened rows.
+#ifndef DISTCA_BWD_KSUB
+#define DISTCA_BWD_KSUB 1
+#endif
+#ifndef DISTCA_BWD_MSUB
+#define DISTCA_BWD_MSUB 1
+#endif
+constexpr int kBwdKsub = DISTCA_BWD_KSUB;
+constexpr int kBwdMsub = DISTCA_BWD_MSUB;
+constexpr int kBwdRows = 32 * kBwdMsub;
+constexpr int kBwdKV = kWaves * 32 * kBwdKsub;
+
+inline int validate_params(const distca_ca_params *p) {
+  if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: this build has kernels for head_dim 128 only", p->head_dim);
+  if (p->num_heads_q <= 0 || p->num_heads_kv <= 0 || p->num_heads_q % p->num_heads_kv)
+    return fail(DISTCA_E_INVALID, "num_heads_q=%d must be a positive multiple of num_heads_kv=%d", p->num_heads_q, p->num_heads_kv);
+  if (p->num_tasks < 0 || p->total_q < 0 || p->total_k < 0 || p->max_seqlen_q < 0 || p->max_seqlen_k < 0)
+    return fail(DISTCA_E_INVALID, "negative size in distca_ca_params");
+  if (!(p->softmax_scale > 0.f) || !isfinite(p->softmax_scale)) return fail(DISTCA_E_INVALID, "softmax_scale must be positive and finite");
+  const int64_t group = p->num_heads_q / p->num_heads_kv;
+  if ((int64_t)p->max_seqlen_q * group >= (1ll << 30) || (int64_t)p->total_q * group >= (1ll << 31))
+    return fail(DISTCA_E_INVALID, "query rows x heads-per-group exceeds 32-bit tile indexing");
+  return DISTCA_OK;
+}
+
+inline SchedGeom fwd_geom(const distca_ca_params *p) {
+  SchedGeom g;
+  g.rows_per_block = kFwdRows;
+  g.kv_per_block = kFwdKV;
+  g.group = p->num_heads_q / p->num_heads_kv;
+  g.causal = p->causal != 0;
+  g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_k / kFwdKV + 1);
+  return g;
+}
+inline SchedGeom bwd_geom(const distca_ca_params *p) {
+  SchedGeom g;
+  g.rows_per_block = kBwdRows;
+  g.kv_per_block = kBwdKV;
+  g.group = p->num_heads_q / p->num_heads_kv;
+  g.causal = p->causal != 0;
+  g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_q * g.group / kBwdRows + 1);
+  return g;
+}
+// Upper bound of the item count that needs only host-known sizes.
+inline int64_t fwd_max_items(const distca_ca_params *p) {
+  const int64_t group = p->num_heads_q / p->num_heads_kv;
+  return (int64_t)p->total_q * group / kFwdRows + p->num_tasks + 1;
+}
+inline int64_t bwd_max_items(const distca_ca_params *p) {
+  // sum over tasks of ceil(Lk / kBwdKV); sum of Lk may exceed total_k when prefixes alias,
+  // but each Lk <= max_seqlen_k.
+  const int64_t by_total = (int64_t)p->total_k / kBwdKV + p->num_tasks + 1;
+  const int64_t by_max = ((int64_t)p->max_seqlen_k / kBwdKV + 1) * p->num_tasks + 1;
+  return by_total > by_max ? by_total : by_max;
+}
+
+int launch_build_schedule(int kind, const int32_t *cu_q, const int32_t *cu_k, int32_t num_tasks, const SchedGeom &g,
+                          int32_t *ws, int64_t max_items, hipStream_t stream);
+
+inline int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace distca

@@ -1,0 +1,347 @@
+// Varlen causal flash-attention forward for gfx950 (wave64, bf16 MFMA 32x32x16).
+//
+// Stands where the reference calls flash-attn's varlen forward
+// (distca/runtime/megatron/ops/fused_comm_attn.py:151-197).
+//
+// Work decomposition.  The G = Hq/Hkv query heads that share a kv head are flattened with
+// the tokens into one row axis: row R of a task = (token R / G, head R % G), so one K/V
+// tile in LDS serves all heads of its group.  A workgroup (4 waves) owns kRows consecutive
+// flattened rows of one task and one kv head and streams that task's visible KV prefix in
+// tiles of 64 keys; tiles entirely above the diagonal are never visited and only tiles
+// that straddle it are masked.
+//
+// Per wave: MSUB sub-tiles of 32 rows.  Scores are produced transposed, S^T = K Q^T, so a
+// lane holds one query row (column lane%32) and 16 keys per 32x32 block: the online-softmax
+// row reductions are in-register plus one lane-pair exchange, and the fp32 accumulator
+// registers are, after conversion to bf16, already laid out as the B operand of
+// O^T += V^T P^T.  Q stays in registers for the whole KV loop; K is read from LDS row-major
+// (16-byte reads), V through the transposing LDS read.
+#include "api_util.h"
+#include "attn_cfg.h"
+#include "common.h"
+
+namespace distca {
+namespace {
+
+constexpr int kKPitch = 272;  // bytes per K row in LDS (256 + 16: rows shift by 4 banks)
+constexpr int kVPitch = 288;  // bytes per V row in LDS (256 + 32: 4 rows x 32 B tile the banks)
+constexpr int kKTile = kFwdKV * kKPitch;
+constexpr int kVTile = kFwdKV * kVPitch;
+constexpr int kStage = kKTile + kVTile;
+constexpr int kFwdLds = 2 * kStage;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct FwdArgs {
+  const __bf16 *q, *k, *v;
+  __bf16 *out;
+  float *lse;
+  const int32_t *cu_q, *cu_k, *kv_off;
+  const int32_t *sched;  // schedule workspace
+  int32_t sched_items_off;  // int32 offset of the item array
+  int32_t hq, hkv, group, total_q;
+  int32_t causal;
+  float scale;
+};
+
+template <int MSUB>
+__global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int nitems = a.sched[0];
+  const int item = blockIdx.x / a.hkv;
+  if (item >= nitems) return;
+  const int kvh = blockIdx.x - item * a.hkv;
+  const int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  const int task = it.x, mblk = it.y;
+
+  const int q0 = a.cu_q[task];
+  const int lq = a.cu_q[task + 1] - q0;
+  const int lk = a.cu_k[task + 1] - a.cu_k[task];
+  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
+  const int G = a.group;
+  const int shift = lk - lq;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  constexpr int kRows = kWaves * 32 * MSUB;
+  const int row_wg = mblk * kRows;
+  const int nrows = lq * G;
+
+  // ---- KV extent of this workgroup
+  int tok_end = (row_wg + kRows + G - 1) / G;
+  if (tok_end > lq) tok_end = lq;
+  int nvis = a.causal ? tok_end + shift : lk;
+  if (nvis > lk) nvis = lk;
+  const int ntiles = nvis > 0 ? (nvis + kFwdKV - 1) / kFwdKV : 0;
+
+  // ---- per-lane rows
+  int row[MSUB], tok[MSUB], lim[MSUB];
+  bool valid[MSUB];
+  const __bf16 *qptr[MSUB];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+    row[m] = row_wg + (wave * MSUB + m) * 32 + l32;
+    valid[m] = row[m] < nrows;
+    tok[m] = row[m] / G;
+    const int hg = row[m] - tok[m] * G;
+    int lm = a.causal ? tok[m] + shift : lk - 1;
+    if (lm > lk - 1) lm = lk - 1;
+    lim[m] = lm;
+    qptr[m] = a.q + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+  }
+  // wave-uniform limits: first row's limit decides whether a tile needs masking, last row's
+  // whether the wave has anything to do in it.
+  const int wrow0 = row_wg + wave * MSUB * 32;
+  int wrow1 = wrow0 + MSUB * 32 - 1;
+  if (wrow1 > nrows - 1) wrow1 = nrows - 1;
+  const bool wave_live = wrow0 < nrows;
+  int lim_first = 0x7fffffff, lim_last = -1;
+  if (wave_live) {
+    lim_first = a.causal ? wrow0 / G + shift : lk - 1;
+    if (lim_first > lk - 1) lim_first = lk - 1;
+    lim_last = a.causal ? wrow1 / G + shift : lk - 1;
+    if (lim_last > lk - 1) lim_last = lk - 1;
+  }
+
+  // ---- Q fragments (B operand of S^T = K Q^T): lane holds row l32, d = 16*s + 8*g .. +7
+  bf16x8 qf[MSUB][8];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (valid[m]) qf[m][s] = *reinterpret_cast<const bf16x8 *>(qptr[m] + 16 * s + 8 * g);
+      else qf[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+
+  // ---- K/V tile staging: 64 rows x 16 chunks of 16 B, 4 chunks per thread
+  const int ld_col = tid & 15;  // 16-byte chunk within the row
+  const int ld_row = tid >> 4;  // + 16*i
+  const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
+  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
+  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
+  u32x4 kreg[4], vreg[4];
+  auto load_tile = [&](int j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = j * kFwdKV + ld_row + 16 * i;
+      if (key < lk) {
+        kreg[i] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)key * kv_stride);
+        vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + (int64_t)key * kv_stride);
+      } else {
+        kreg[i] = u32x4{0, 0, 0, 0};
+        vreg[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto store_tile = [&](int stage) {
+    uint8_t *kt = lds + stage * kStage;
+    uint8_t *vt = kt + kKTile;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = ld_row + 16 * i;
+      *reinterpret_cast<u32x4 *>(kt + r * kKPitch + ld_col * 16) = kreg[i];
+      *reinterpret_cast<u32x4 *>(vt + r * kVPitch + ld_col * 16) = vreg[i];
+    }
+  };
+
+  // ---- accumulators
+  f32x16 oacc[MSUB][4];
+  float m_run[MSUB], l_run[MSUB];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[m][db][r] = 0.f;
+    m_run[m] = -INFINITY;
+    l_run[m] = 0.f;
+  }
+  const float c = a.scale * kLog2e;
+
+  // LDS read offsets (bytes) that do not depend on the tile
+  const int k_rd = l32 * kKPitch + 16 * g;                                            // + kb*32*kKPitch + 32*s
+  const int v_rd = (4 * g + ((lane & 15) >> 2)) * kVPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // + (16t+8h)*kVPitch + 32*db
+
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int stage = j & 1;
+    const uint8_t *kt = lds + stage * kStage;
+    const uint8_t *vt = kt + kKTile;
+    const bool has_next = j + 1 < ntiles;
+    if (has_next) load_tile(j + 1);
+
+    const int key0 = j * kFwdKV;
+    const bool active = wave_live && key0 <= lim_last;
+    bf16x8 pf[MSUB][4];
+    if (active) {
+      // ---- S^T = K Q^T : [64 keys] x [32*MSUB rows]
+      f32x16 sacc[MSUB][2];
+#pragma unroll
+      for (int m = 0; m < MSUB; ++m)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[m][kb][r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(kt + k_rd + kb * 32 * kKPitch + 32 * s);
+#pragma unroll
+          for (int m = 0; m < MSUB; ++m) sacc[m][kb] = mfma32(kf, qf[m][s], sacc[m][kb]);
+        }
+      }
+      // ---- mask the tiles that straddle the diagonal or the end of the prefix
+      if (key0 + kFwdKV - 1 > lim_first) {
+#pragma unroll
+        for (int m = 0; m < MSUB; ++m)
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = key0 + kb * 32 + acc_row(r, g);
+              if (key > lim[m]) sacc[m][kb][r] = -INFINITY;
+            }
+      }
+      // ---- online softmax (log2 domain), one query row per lane pair
+#pragma unroll
+      for (int m = 0; m < MSUB; ++m) {
+        float mx = sacc[m][0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, sacc[m][kb][r]);
+        mx = pair_max(mx);
+        const float m_new = __builtin_fmaxf(m_run[m], mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        if (__any(m_new != m_run[m])) {
+          const float alpha = fast_exp2((m_run[m] - m_use) * c);
+          l_run[m] *= alpha;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[m][db][r] *= alpha;
+          m_run[m] = m_new;
+        }
+        const float mc = -m_use * c;
+        float sum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, mc));
+            sacc[m][kb][r] = p;
+            sum += p;
+          }
+        l_run[m] += sum;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int kb = t >> 1, r0 = 8 * (t & 1);
+          pf[m][t] = cvt8(sacc[m][kb][r0], sacc[m][kb][r0 + 1], sacc[m][kb][r0 + 2], sacc[m][kb][r0 + 3], sacc[m][kb][r0 + 4],
+                          sacc[m][kb][r0 + 5], sacc[m][kb][r0 + 6], sacc[m][kb][r0 + 7]);
+        }
+      }
+    }
+    // ---- next tile into the other LDS stage (its last readers finished before the
+    //      barrier that ended the previous iteration)
+    if (has_next) store_tile(stage ^ 1);
+
+    if (active) {
+      // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const uint8_t *vp = vt + v_rd + 16 * t * kVPitch + 32 * db;
+          const bf16x4 lo = lds_read_tr((const DISTCA_LDS void *)vp);
+          const bf16x4 hi = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kVPitch));
+          const bf16x8 vf = cat4(lo, hi);
+#pragma unroll
+          for (int m = 0; m < MSUB; ++m) oacc[m][db] = mfma32(vf, pf[m][t], oacc[m][db]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise, write O (bf16) and LSE (fp32, natural log)
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+    const float l_tot = pair_sum(l_run[m]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (valid[m]) {
+      const int hg = row[m] - tok[m] * G;
+      __bf16 *op = a.out + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int cq = 0; cq < 4; ++cq) {
+          // registers 4*cq .. 4*cq+3 of block db hold d0 .. d0+3
+          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
+          const bf16x4 o4 = cvt4(oacc[m][db][4 * cq] * inv, oacc[m][db][4 * cq + 1] * inv, oacc[m][db][4 * cq + 2] * inv,
+                                 oacc[m][db][4 * cq + 3] * inv);
+          *reinterpret_cast<bf16x4 *>(op + d0) = o4;
+        }
+      if (g == 0) {
+        const float lse = l_tot > 0.f ? (m_run[m] * c + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]] = lse;
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace distca
+
+using namespace distca;
+
+extern "C" int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p) {
+  if (!p) return fail(DISTCA_E_INVALID, "fwd_workspace_bytes: null params");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  return align_up(sched_bytes(p->num_tasks, fwd_max_items(p)), 256);
+}
+
+extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
+                             const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
+                             int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
+  if (!q || !k || !v || !out || !lse || !cu_q || !cu_k) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return fail(DISTCA_E_INVALID, "ca_fwd: q/k/v/out must be 16-byte aligned");
+  const int64_t need = distca_ca_fwd_workspace_bytes(p);
+  if (!workspace || workspace_bytes < need) return fail(DISTCA_E_WORKSPACE, "ca_fwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)need);
+  if (!aligned16(workspace)) return fail(DISTCA_E_INVALID, "ca_fwd: workspace must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const SchedGeom geom = fwd_geom(p);
+  const int64_t max_items = fwd_max_items(p);
+  rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)workspace, max_items, s);
+  if (rc) return rc;
+
+  FwdArgs a;
+  a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v;
+  a.out = (__bf16 *)out; a.lse = lse;
+  a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
+  a.sched = (const int32_t *)workspace;
+  a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
+  a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
+  a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
+  const int64_t grid = max_items * p->num_heads_kv;
+  if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
+    if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kFwdLds, s, a);
+  return check_launch("ca_fwd");
+}

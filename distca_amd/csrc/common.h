@@ -1,0 +1,62 @@
+// Shared device helpers for the gfx950 core-attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace distca {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define DISTCA_LDS __attribute__((address_space(3)))
+
+// D = A(32x16) * B(16x32) + C on one wave64.
+//   A operand: lane l holds row l%32, k = 8*(l/32) .. +7
+//   B operand: lane l holds col l%32, k = 8*(l/32) .. +7
+//   C/D:       lane l holds col l%32, register r holds row 8*(r/4) + 4*(l/32) + r%4
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Row index (0..31) inside a 32x32 accumulator block for register r of lane-half g.
+__device__ __forceinline__ constexpr int acc_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
+// Transposing LDS read.  Within each group of 16 lanes, lane j supplies the address of
+// 4 consecutive 16-bit elements; lane L of the group receives element (L%4) of the
+// chunks supplied by lanes 4e + L/4, e = 0..3.  With lane j pointing at
+// (row r0 + j/4, col c0 + 4*(j%4)) of a row-major tile, lane L ends up with
+// column c0 + L of rows r0 .. r0+3.
+__device__ __forceinline__ bf16x4 lds_read_tr(const DISTCA_LDS void *p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DISTCA_LDS s16x4 *)p);
+  return __builtin_bit_cast(bf16x4, v);
+}
+
+__device__ __forceinline__ bf16x8 cat4(bf16x4 lo, bf16x4 hi) {
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ bf16x8 cvt8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
+  f32x8 v = {a0, a1, a2, a3, a4, a5, a6, a7};
+  return __builtin_convertvector(v, bf16x8);
+}
+__device__ __forceinline__ bf16x4 cvt4(float a0, float a1, float a2, float a3) {
+  f32x4 v = {a0, a1, a2, a3};
+  return __builtin_convertvector(v, bf16x4);
+}
+
+// max / sum of x over the lane pair (l, l^32).
+__device__ __forceinline__ float pair_max(float x) { return __builtin_fmaxf(x, __shfl_xor(x, 32, 64)); }
+__device__ __forceinline__ float pair_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+}  // namespace distca

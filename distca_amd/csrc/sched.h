@@ -1,0 +1,86 @@
+// Tile scheduler: turns (cu_seqlens_q, cu_seqlens_k) into a list of work items sorted by
+// descending cost.  The attention kernels are launched with one workgroup per
+// (item, kv-head) in list order, workgroup id = item_rank * Hkv + kv_head.  The hardware
+// dispatcher hands workgroups to compute units in id order as slots free up, so a sorted
+// list gives longest-processing-time-first balancing across CUs without a persistent
+// kernel or atomics; and because workgroup ids are dealt round-robin over the 8 XCDs,
+// with Hkv = 8 every XCD works on one kv head and its L2 holds only that head's K/V.
+//
+// Cost unit = the causal-pair count the reference's planner balances across ranks
+// (Item.get_flops, distca/planner/planner.py:366-378), here at tile granularity.
+// The reference itself has no such component on the GPU: flash-attn launches a static
+// (m-block, batch, head) grid sized by max_seqlen_q.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define DISTCA_HD __host__ __device__ __forceinline__
+#else
+#define DISTCA_HD inline
+#endif
+
+namespace distca {
+
+struct SchedGeom {
+  int32_t rows_per_block;  // flattened (token, head-in-group) query rows per m-block
+  int32_t kv_per_block;    // keys per KV block
+  int32_t group;           // Hq / Hkv
+  int32_t causal;
+  int32_t cost_shift;      // bin = min(kSchedBins-1, cost >> cost_shift)
+};
+
+constexpr int kSchedBins = 4096;
+
+DISTCA_HD int32_t ceil_div(int32_t a, int32_t b) { return (a + b - 1) / b; }
+
+// forward: blocks of query rows
+DISTCA_HD int32_t fwd_num_blocks(const SchedGeom &g, int32_t lq) { return ceil_div(lq * g.group, g.rows_per_block); }
+
+// Keys visible to the last token of m-block i (0 when none): the KV extent the block streams.
+DISTCA_HD int32_t fwd_visible_keys(const SchedGeom &g, int32_t lq, int32_t lk, int32_t i) {
+  int32_t tok_end = ceil_div((i + 1) * g.rows_per_block, g.group);  // one past the last token
+  if (tok_end > lq) tok_end = lq;
+  int32_t nvis = g.causal ? tok_end + (lk - lq) : lk;
+  if (nvis > lk) nvis = lk;
+  return nvis > 0 ? nvis : 0;
+}
+DISTCA_HD int32_t fwd_cost(const SchedGeom &g, int32_t lq, int32_t lk, int32_t i) {
+  return ceil_div(fwd_visible_keys(g, lq, lk, i), g.kv_per_block);
+}
+
+// backward: blocks of keys
+DISTCA_HD int32_t bwd_num_blocks(const SchedGeom &g, int32_t lq, int32_t lk) {
+  return lq > 0 ? ceil_div(lk, g.kv_per_block) : 0;
+}
+// First m-block that sees any key of KV block n.
+DISTCA_HD int32_t bwd_first_mblock(const SchedGeom &g, int32_t lq, int32_t lk, int32_t n) {
+  if (!g.causal) return 0;
+  int32_t t_first = n * g.kv_per_block - (lk - lq);
+  if (t_first < 0) t_first = 0;
+  return (int32_t)(((int64_t)t_first * g.group) / g.rows_per_block);
+}
+DISTCA_HD int32_t bwd_cost(const SchedGeom &g, int32_t lq, int32_t lk, int32_t n) {
+  int32_t c = fwd_num_blocks(g, lq) - bwd_first_mblock(g, lq, lk, n);
+  return c > 0 ? c : 0;
+}
+
+DISTCA_HD int32_t cost_bin(const SchedGeom &g, int32_t cost) {
+  int32_t b = cost >> g.cost_shift;
+  return b < kSchedBins - 1 ? b : kSchedBins - 1;
+}
+
+inline int32_t pick_cost_shift(int64_t max_cost) {
+  int32_t s = 0;
+  while ((max_cost >> s) >= kSchedBins) ++s;
+  return s;
+}
+
+// Workspace layout of a schedule (all int32):
+//   [0] item count   [1..3] reserved   [4 .. 4+B] exclusive block prefix per task
+//   then items as (task, block, cost, 0) quadruples, 16-byte aligned.
+DISTCA_HD int64_t sched_header_ints(int32_t num_tasks) { return ((int64_t)4 + num_tasks + 1 + 3) / 4 * 4; }
+DISTCA_HD int64_t sched_bytes(int32_t num_tasks, int64_t max_items) {
+  return (sched_header_ints(num_tasks) + 4 * max_items) * (int64_t)sizeof(int32_t);
+}
+
+}  // namespace distca

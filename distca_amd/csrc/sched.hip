@@ -1,0 +1,176 @@
+// Device builder and host mirror of the tile schedule described in sched.h.
+#include <algorithm>
+#include <vector>
+
+#include "api_util.h"
+#include "attn_cfg.h"
+#include "sched.h"
+
+namespace distca {
+namespace {
+
+constexpr int kSchedThreads = 1024;
+
+__device__ __forceinline__ int32_t block_inclusive_scan_i32(int32_t v, int32_t *wave_sums) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int32_t o = __shfl_up(v, off, 64);
+    if (lane >= off) v += o;
+  }
+  __syncthreads();
+  if (lane == 63) wave_sums[wave] = v;
+  __syncthreads();
+  int32_t base = 0;
+  for (int w = 0; w < wave; ++w) base += wave_sums[w];
+  return v + base;
+}
+
+template <bool BWD>
+__device__ __forceinline__ int32_t item_cost(const SchedGeom &g, const int32_t *cu_q, const int32_t *cu_k, int32_t b, int32_t i) {
+  const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
+  return BWD ? bwd_cost(g, lq, lk, i) : fwd_cost(g, lq, lk, i);
+}
+
+// Largest b in [0, B) with base[b] <= e.
+__device__ __forceinline__ int32_t find_task(const int32_t *base, int32_t num_tasks, int32_t e) {
+  int32_t lo = 0, hi = num_tasks;  // invariant: base[lo] <= e < base[hi]
+  while (hi - lo > 1) {
+    int32_t mid = (lo + hi) >> 1;
+    if (base[mid] <= e) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+template <bool BWD>
+__global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int32_t *__restrict__ cu_q,
+                                                                     const int32_t *__restrict__ cu_k, int32_t num_tasks,
+                                                                     SchedGeom g, int32_t *__restrict__ ws, int32_t max_items) {
+  __shared__ int32_t bins[kSchedBins];
+  __shared__ int32_t wave_sums[kSchedThreads / 64];
+  __shared__ int32_t carry;
+  int32_t *base = ws + 4;
+  int32_t *items = ws + sched_header_ints(num_tasks);
+  const int tid = threadIdx.x;
+
+  // 1. exclusive prefix of block counts per task
+  int32_t running = 0;
+  for (int32_t c0 = 0; c0 < num_tasks; c0 += kSchedThreads) {
+    const int32_t b = c0 + tid;
+    int32_t n = 0;
+    if (b < num_tasks) {
+      const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
+      n = BWD ? bwd_num_blocks(g, lq, lk) : fwd_num_blocks(g, lq);
+      if (n < 0) n = 0;
+    }
+    const int32_t incl = block_inclusive_scan_i32(n, wave_sums);
+    if (b < num_tasks) base[b] = running + incl - n;
+    __syncthreads();
+    if (tid == kSchedThreads - 1) carry = running + incl;
+    __syncthreads();
+    running = carry;
+  }
+  int32_t nitems = running < max_items ? running : max_items;
+  if (tid == 0) base[num_tasks] = running;
+  for (int i = tid; i < kSchedBins; i += kSchedThreads) bins[i] = 0;
+  __syncthreads();
+
+  // 2. histogram of cost bins
+  for (int32_t e = tid; e < nitems; e += kSchedThreads) {
+    const int32_t b = find_task(base, num_tasks, e);
+    const int32_t cost = item_cost<BWD>(g, cu_q, cu_k, b, e - base[b]);
+    atomicAdd(&bins[cost_bin(g, cost)], 1);
+  }
+  __syncthreads();
+
+  // 3. start offset of each bin when bins are laid out from the most expensive down
+  {
+    constexpr int kPer = kSchedBins / kSchedThreads;
+    int32_t cnt[kPer], local = 0;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      cnt[u] = bins[kSchedBins - 1 - (tid * kPer + u)];
+      local += cnt[u];
+    }
+    const int32_t incl = block_inclusive_scan_i32(local, wave_sums);
+    int32_t start = incl - local;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      bins[kSchedBins - 1 - (tid * kPer + u)] = start;
+      start += cnt[u];
+    }
+  }
+  __syncthreads();
+
+  // 4. scatter
+  for (int32_t e = tid; e < nitems; e += kSchedThreads) {
+    const int32_t b = find_task(base, num_tasks, e);
+    const int32_t i = e - base[b];
+    const int32_t cost = item_cost<BWD>(g, cu_q, cu_k, b, i);
+    const int32_t pos = atomicAdd(&bins[cost_bin(g, cost)], 1);
+    if (pos < max_items) {
+      int4 it = make_int4(b, i, cost, 0);
+      reinterpret_cast<int4 *>(items)[pos] = it;
+    }
+  }
+  if (tid == 0) {
+    ws[0] = nitems;
+    ws[1] = running;
+  }
+}
+
+}  // namespace
+
+int launch_build_schedule(int kind, const int32_t *cu_q, const int32_t *cu_k, int32_t num_tasks, const SchedGeom &g,
+                          int32_t *ws, int64_t max_items, hipStream_t stream) {
+  if (max_items > 0x7fffffff) return fail(DISTCA_E_INVALID, "schedule: too many work items");
+  if (kind == 0)
+    hipLaunchKernelGGL((build_schedule_kernel<false>), dim3(1), dim3(kSchedThreads), 0, stream, cu_q, cu_k, num_tasks, g, ws,
+                       (int32_t)max_items);
+  else
+    hipLaunchKernelGGL((build_schedule_kernel<true>), dim3(1), dim3(kSchedThreads), 0, stream, cu_q, cu_k, num_tasks, g, ws,
+                       (int32_t)max_items);
+  return check_launch("build_schedule");
+}
+
+}  // namespace distca
+
+using namespace distca;
+
+extern "C" int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]) {
+  if (!p || !out) return fail(DISTCA_E_INVALID, "tile_shape: null pointer");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  SchedGeom g = kind == 0 ? fwd_geom(p) : bwd_geom(p);
+  out[0] = g.rows_per_block;  // flattened (token, head-in-group) rows
+  out[1] = g.kv_per_block;
+  return DISTCA_OK;
+}
+
+extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const int32_t *cu_k, const distca_ca_params *p,
+                                           int32_t *items, int64_t max_items) {
+  if (!p || !cu_q || !cu_k || (!items && max_items > 0)) return fail(DISTCA_E_INVALID, "schedule_host: null pointer");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  if (kind != 0 && kind != 1) return fail(DISTCA_E_INVALID, "schedule_host: kind must be 0 (fwd) or 1 (bwd)");
+  const SchedGeom g = kind == 0 ? fwd_geom(p) : bwd_geom(p);
+  struct It { int32_t task, block, cost, bin; };
+  std::vector<It> v;
+  for (int32_t b = 0; b < p->num_tasks; ++b) {
+    const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
+    const int32_t n = kind == 0 ? fwd_num_blocks(g, lq) : bwd_num_blocks(g, lq, lk);
+    for (int32_t i = 0; i < n; ++i) {
+      const int32_t c = kind == 0 ? fwd_cost(g, lq, lk, i) : bwd_cost(g, lq, lk, i);
+      v.push_back({b, i, c, cost_bin(g, c)});
+    }
+  }
+  std::stable_sort(v.begin(), v.end(), [](const It &a, const It &b) { return a.bin > b.bin; });
+  const int64_t n = (int64_t)v.size();
+  for (int64_t e = 0; e < n && e < max_items; ++e) {
+    items[3 * e + 0] = v[e].task;
+    items[3 * e + 1] = v[e].block;
+    items[3 * e + 2] = v[e].cost;
+  }
+  return n;
+}

@@ -1,0 +1,301 @@
+"""The CA server's attention ops: unpack -> varlen core attention -> pack.
+
+Mirrors distca/runtime/megatron/ops/fused_comm_attn.py: FlashAttnArgs (:80-104),
+_qkv_to_attn_out_fwd (:108-201), _qkv_to_attn_out_bwd (:204-279) and the ordering of
+FusedCommAttn.forward / backward (:287-461).  The flash-attn calls of the reference are
+replaced by distca_ca_fwd / distca_ca_bwd of the C ABI (hand-written gfx950 kernels);
+there is no other attention implementation behind these functions.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .dispatch import (post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_with_lse, pre_a2a_qkv)
+
+
+@dataclass
+class PackedSeqParams:
+    """The fields of megatron's PackedSeqParams the CA server reads
+    (distca/runtime/megatron/packed_seq_params.py:26-57): int32 device cu_seqlens and
+    Python-int max_seqlen.  `kv_task_offsets` (int32 [B], optional) gives the first KV row
+    of every task so that tasks of one document can share a single KV prefix instead of
+    holding one copy each; omitted, task b reads rows cu_seqlens_kv[b]..cu_seqlens_kv[b+1]."""
+    cu_seqlens_q: Tensor = None
+    cu_seqlens_kv: Tensor = None
+    max_seqlen_q: int = None
+    max_seqlen_kv: int = None
+    qkv_format: str = "thd"
+    kv_task_offsets: Optional[Tensor] = None
+
+
+@dataclass
+class FlashAttnArgs:
+    num_heads_q: int
+    num_heads_kv: int
+    head_dim: int
+    dropout_p: float = 0.0
+    softmax_scale: float = None
+    causal: bool = True
+    window_size: Tuple[int, int] = (-1, -1)
+    softcap: float = 0.0
+    alibi_slopes = None
+    deterministic: bool = None
+    return_attn_probs: bool = False
+    block_table = None
+
+    def __post_init__(self):
+        if self.deterministic is None:
+            # same switch as the reference (fused_comm_attn.py:95-104)
+            self.deterministic = os.getenv("NVTE_ALLOW_NONDETERMINISTIC_ALGO", "0") != "1"
+
+
+def _params(num_tasks, total_q, total_k, hq, hkv, d, max_q, max_k, scale, causal, deterministic) -> _lib.CaParams:
+    return _lib.CaParams(num_tasks, total_q, total_k, hq, hkv, d, int(max_q), int(max_k), float(scale),
+                         1 if causal else 0, 1 if deterministic else 0, 0)
+
+
+def _check_qkv(q: Tensor, k: Tensor, v: Tensor, cu_q: Tensor, cu_k: Tensor, kv_off: Optional[Tensor]):
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dim() != 3:
+            raise RuntimeError(f"{name} must have shape [tokens, heads, head_dim]")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be on CUDA")
+        if t.dtype != torch.bfloat16:
+            raise RuntimeError(f"{name} must be bfloat16 (got {t.dtype})")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    if k.shape != v.shape:
+        raise RuntimeError("k and v must have the same shape")
+    if q.shape[2] != k.shape[2]:
+        raise RuntimeError("q and k must have the same head_dim")
+    for name, t in (("cu_seqlens_q", cu_q), ("cu_seqlens_k", cu_k)):
+        if t.dtype != torch.int32 or not t.is_cuda or t.dim() != 1 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous 1-D int32 CUDA tensor")
+    if cu_q.shape != cu_k.shape:
+        raise RuntimeError("cu_seqlens_q and cu_seqlens_k must have the same shape")
+    if kv_off is not None:
+        if kv_off.dtype != torch.int32 or not kv_off.is_cuda or kv_off.shape[0] != cu_q.shape[0] - 1:
+            raise RuntimeError("kv_task_offsets must be an int32 CUDA tensor of shape [num_tasks]")
+
+
+def ca_varlen_fwd(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor, cu_seqlens_k: Tensor,
+                  max_seqlen_q: int, max_seqlen_k: int, softmax_scale: Optional[float] = None, causal: bool = True,
+                  kv_task_offsets: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """q [Tq,Hq,D], k,v [Tk,Hkv,D] bf16 -> (out [Tq,Hq,D] bf16, softmax_lse [Hq,Tq] fp32)."""
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
+    tq, hq, d = q.shape
+    tk, hkv, _ = k.shape
+    scale = softmax_scale if softmax_scale is not None else d ** (-0.5)
+    lib = _lib.load()
+    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, False)
+    need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
+    if need < 0:
+        _lib.check(int(need), "ca_varlen_fwd")
+    out = torch.empty_like(q)
+    lse = torch.empty((hq, tq), dtype=torch.float32, device=q.device)
+    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.distca_ca_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                               cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                               kv_task_offsets.data_ptr() if kv_task_offsets is not None else None,
+                               ctypes.byref(p), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ca_varlen_fwd")
+    return out, lse
+
+
+def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, softmax_lse: Tensor,
+                  cu_seqlens_q: Tensor, cu_seqlens_k: Tensor, max_seqlen_q: int, max_seqlen_k: int,
+                  softmax_scale: Optional[float] = None, causal: bool = True, deterministic: bool = False,
+                  kv_task_offsets: Optional[Tensor] = None,
+                  dq: Optional[Tensor] = None, dk: Optional[Tensor] = None, dv: Optional[Tensor] = None):
+    """Gradients (dq, dk, dv) in bf16; written into dq/dk/dv when given (the reference's
+    flash-attn backward fills caller-allocated tensors, fused_comm_attn.py:236,259-272)."""
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
+    tq, hq, d = q.shape
+    tk, hkv, _ = k.shape
+    for name, t in (("dout", dout), ("out", out)):
+        if t.shape != q.shape or t.dtype != torch.bfloat16 or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a bfloat16 CUDA tensor shaped like q")
+    dout = dout.contiguous()
+    out = out.contiguous()
+    if softmax_lse.shape != (hq, tq) or softmax_lse.dtype != torch.float32:
+        raise RuntimeError(f"softmax_lse must be fp32 of shape [Hq, Tq] = {(hq, tq)}, got {tuple(softmax_lse.shape)}")
+    softmax_lse = softmax_lse.contiguous()
+    scale = softmax_scale if softmax_scale is not None else d ** (-0.5)
+    lib = _lib.load()
+    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, deterministic)
+    need = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+    if need < 0:
+        _lib.check(int(need), "ca_varlen_bwd")
+    dq = torch.empty_like(q) if dq is None else dq
+    dk = torch.empty_like(k) if dk is None else dk
+    dv = torch.empty_like(v) if dv is None else dv
+    for name, t, ref in (("dq", dq, q), ("dk", dk, k), ("dv", dv, v)):
+        if t.shape != ref.shape or t.dtype != torch.bfloat16 or not t.is_contiguous() or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a contiguous bfloat16 CUDA tensor shaped like its input")
+    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.distca_ca_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                               softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                               cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                               kv_task_offsets.data_ptr() if kv_task_offsets is not None else None,
+                               ctypes.byref(p), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ca_varlen_bwd")
+    return dq, dk, dv
+
+
+def _qkv_to_attn_out_fwd(q: Tensor, k: Tensor, v: Tensor, fa_params: PackedSeqParams, fa_args: FlashAttnArgs):
+    """2-D [T, H*D] q/k/v in, (out [T, Hq*D], softmax_lse [Hq, T]) out — the contract of
+    fused_comm_attn.py:108-201."""
+    assert fa_args.causal
+    assert fa_args.window_size == (-1, -1)
+    assert fa_args.alibi_slopes is None
+    assert fa_args.block_table is None
+    assert fa_args.dropout_p == 0.0
+    q = q.reshape(q.shape[0], fa_args.num_heads_q, fa_args.head_dim)
+    k = k.reshape(k.shape[0], fa_args.num_heads_kv, fa_args.head_dim)
+    v = v.reshape(v.shape[0], fa_args.num_heads_kv, fa_args.head_dim)
+    softmax_scale = fa_args.softmax_scale
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    out, softmax_lse = ca_varlen_fwd(
+        q.contiguous(), k.contiguous(), v.contiguous(), fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
+        fa_params.max_seqlen_q, fa_params.max_seqlen_kv, softmax_scale, causal=fa_args.causal,
+        kv_task_offsets=getattr(fa_params, "kv_task_offsets", None))
+    out = out.reshape(out.shape[0], fa_args.num_heads_q * fa_args.head_dim)
+    return out, softmax_lse
+
+
+def _qkv_to_attn_out_bwd(
+    q: Tensor, k: Tensor, v: Tensor, attn_out: Tensor,
+    attn_out_grad: Tensor, softmax_lse: Tensor,
+    fa_args: FlashAttnArgs, cu_seqlen_q: Tensor, cu_seqlen_kv: Tensor,
+    max_seqlen_q: int, max_seqlen_kv: int, kv_task_offsets: Optional[Tensor] = None,
+):
+    """(dq [T,Hq*D], dk, dv [Tk,Hkv*D]) — the contract of fused_comm_attn.py:204-279;
+    softmax_lse is [Hq, T]."""
+    hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
+    q = q.reshape(q.shape[0], hq, d).contiguous()
+    k = k.reshape(k.shape[0], hkv, d).contiguous()
+    v = v.reshape(v.shape[0], hkv, d).contiguous()
+    out = attn_out.reshape(attn_out.shape[0], hq, d)
+    dout = attn_out_grad.reshape(attn_out_grad.shape[0], hq, d)
+    softmax_scale = fa_args.softmax_scale
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    dq, dk, dv = ca_varlen_bwd(dout, q, k, v, out, softmax_lse, cu_seqlen_q, cu_seqlen_kv, max_seqlen_q, max_seqlen_kv,
+                               softmax_scale, fa_args.causal, fa_args.deterministic, kv_task_offsets)
+    return (dq.reshape(dq.shape[0], hq * d), dk.reshape(dk.shape[0], hkv * d), dv.reshape(dv.shape[0], hkv * d))
+
+
+class CoreAttention(torch.autograd.Function):
+    """Differentiable varlen core attention on [T, H, D] tensors (drop-in for
+    flash_attn_varlen_func(..., causal=True) on the reference's call pattern)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
+                deterministic, kv_task_offsets):
+        out, lse = ca_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
+                                 kv_task_offsets)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k)
+        ctx.kv_task_offsets = kv_task_offsets
+        ctx.args = (max_seqlen_q, max_seqlen_k, softmax_scale, causal, deterministic)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, cu_q, cu_k = ctx.saved_tensors
+        max_q, max_k, scale, causal, det = ctx.args
+        dq, dk, dv = ca_varlen_bwd(dout.contiguous(), q, k, v, out, lse, cu_q, cu_k, max_q, max_k, scale, causal, det,
+                                   ctx.kv_task_offsets)
+        return dq, dk, dv, None, None, None, None, None, None, None, None
+
+
+def core_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale=None, causal=True,
+                   deterministic=False, kv_task_offsets=None):
+    return CoreAttention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
+                               deterministic, kv_task_offsets)
+
+
+# ---------------------------------------------------------------------------------------
+# The CA server tick, with explicit buffers: what FusedCommAttn.forward / backward do
+# between "receive buffer holds this tick's shards" and "send buffer holds the reply".
+# ---------------------------------------------------------------------------------------
+@dataclass
+class ServerFwdMeta:
+    """Receive-side layout of q/k/v shards and send-side layout of the reply."""
+    q_recv_seq_tokens: Tensor      # int64 [nq_shards]
+    k_recv_seq_tokens: Tensor      # int64 [nk_shards]
+    q_recv_offset: Tensor          # int64 byte offsets into the receive buffer
+    k_recv_offset: Tensor
+    v_recv_offset: Tensor
+    out_send_seq_tokens: Tensor    # int64 [nq_shards]
+    out_send_offset: Tensor        # int64 byte offsets into the send buffer ([out | lse] tokens)
+    recv_q_shape: Tuple[int, int]  # (Tq, Hq*D)
+    recv_k_shape: Tuple[int, int]  # (Tk, Hkv*D)
+
+
+def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdMeta, fa_params: PackedSeqParams,
+                      fa_args: FlashAttnArgs, dtype: torch.dtype = torch.bfloat16):
+    """fused_comm_attn.py:298-389: unpack q,k,v -> attention -> pack [out | lse].
+    Returns (attn_out [T,Hq*D], softmax_lse [Hq,T]) as well, for the caller's own use."""
+    dev = recv_buffer.device
+    recv_q = torch.empty(meta.recv_q_shape, dtype=dtype, device=dev)
+    recv_k = torch.empty(meta.recv_k_shape, dtype=dtype, device=dev)
+    recv_v = torch.empty_like(recv_k)
+    post_a2a_qkv(recv_q, recv_k, recv_v, None, meta.q_recv_seq_tokens, meta.k_recv_seq_tokens,
+                 meta.q_recv_offset, meta.k_recv_offset, meta.v_recv_offset, is_fwd=True, buffer=recv_buffer)
+    attn_out, softmax_lse = _qkv_to_attn_out_fwd(recv_q, recv_k, recv_v, fa_params, fa_args)
+    lse_t = softmax_lse.T.contiguous()  # [T, Hq] for transport (fused_comm_attn.py:370-371)
+    pre_a2a_attn_out_with_lse(attn_out, lse_t, meta.out_send_seq_tokens, meta.out_send_offset, buffer=send_buffer)
+    return attn_out, softmax_lse
+
+
+@dataclass
+class ServerBwdMeta:
+    q_recv_seq_tokens: Tensor      # merged [dO | O | lse | q] shards
+    k_recv_seq_tokens: Tensor
+    q_recv_offset: Tensor
+    k_recv_offset: Tensor
+    v_recv_offset: Tensor
+    q_grad_send_seq_tokens: Tensor
+    k_grad_send_seq_tokens: Tensor
+    q_grad_send_offset: Tensor
+    k_grad_send_offset: Tensor
+    v_grad_send_offset: Tensor
+    main_copy_mask: Tensor         # int8 [nk_shards]
+    num_copies: Tensor             # int32 [nk_shards]
+    copy_start_id: Tensor          # int64 [nk_shards, max_copies]
+    attn_out_shape: Tuple[int, int]
+    lse_shape: Tuple[int, int]     # (T, Hq)
+    k_shape: Tuple[int, int]
+
+
+def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwdMeta, fa_args: FlashAttnArgs,
+                       cu_seqlens_q: Tensor, cu_seqlens_kv: Tensor, max_seqlen_q: int, max_seqlen_kv: int,
+                       dtype: torch.dtype = torch.bfloat16):
+    """fused_comm_attn.py:407-461: unpack merged request -> attention backward -> sum
+    duplicate KV gradients -> masked pack of dq, dk, dv."""
+    dev = recv_buffer.device
+    recv_k = torch.empty(meta.k_shape, dtype=dtype, device=dev)
+    recv_v = torch.empty_like(recv_k)
+    (dout, out, lse, q, recv_k, recv_v) = post_a2a_attn_out_grad_resend_qkv(
+        meta.attn_out_shape, meta.lse_shape, meta.attn_out_shape, torch.float32, recv_k, recv_v, None,
+        meta.q_recv_seq_tokens, meta.k_recv_seq_tokens, meta.q_recv_offset, meta.k_recv_offset, meta.v_recv_offset,
+        is_fwd=True, buffer=recv_buffer)
+    lse = lse.T.contiguous()  # [Hq, T] (fused_comm_attn.py:440)
+    dq, dk, dv = _qkv_to_attn_out_bwd(q, recv_k, recv_v, out, dout, lse, fa_args, cu_seqlens_q, cu_seqlens_kv,
+                                      max_seqlen_q, max_seqlen_kv)
+    dq, dk, dv = pre_a2a_qkv(
+        dq, dk, dv, None, meta.q_grad_send_seq_tokens, meta.k_grad_send_seq_tokens,
+        meta.q_grad_send_offset, meta.k_grad_send_offset, meta.v_grad_send_offset,
+        is_fwd=False, kv_grad_copy_shard_mask=meta.main_copy_mask,
+        pre_a2a_grad_acc_args=(meta.num_copies, meta.copy_start_id, meta.k_grad_send_seq_tokens), buffer=send_buffer)
+    return dq, dk, dv

@@ -1,0 +1,140 @@
+"""Shard pack / unpack / duplicate-gradient ops of the CA server.
+
+Same names, argument order and error behaviour as the reference's Python wrappers
+(distca/runtime/attn_kernels/ops.py:153-215), bound to the HIP kernels through the C ABI
+instead of torch.ops.dispatch_kernels.  The reference can take its transport buffer from
+an NVSHMEM dispatcher; here the buffer is always an explicit device tensor (the
+reference's `buffer=` form, csrc/bindings/all_to_all.cpp:102-113,243-254): on one GPU a
+task buffer is ordinary device memory.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _check_tensor(ndim: int, x: torch.Tensor, name: str) -> None:
+    # mirrors _CHECK_TENSOR, csrc/bindings/all_to_all.cpp:18-21
+    if x.dim() != ndim:
+        raise RuntimeError(f"tensor {name} must have {ndim} dimensions")
+    if not x.is_cuda:
+        raise RuntimeError(f"tensor {name} must be on CUDA")
+    if not x.is_contiguous():
+        raise RuntimeError(f"tensor {name} must be contiguous")
+
+
+def _check_dtype(x: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    # the reference reads metadata through const_data_ptr<T>(), which throws on a mismatch
+    if x.dtype != dtype:
+        raise RuntimeError(f"expected scalar type {dtype} but found {x.dtype} for {name}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def a2a_memcpy_non_cp(
+    tensor: torch.Tensor, nvshmem_offset: torch.Tensor,
+    shard_tokens: torch.Tensor, to_nvshmem: bool,
+    shard_do_copy_mask: Optional[torch.Tensor] = None,
+    buffer: Optional[torch.Tensor] = None, instance_id: Optional[int] = None,
+):
+    """Pack (`to_nvshmem=True`) rows of `tensor` [T, hidden] into `buffer`, or unpack them.
+
+    Shard s covers rows excl_cumsum(shard_tokens)[s].. and buffer bytes nvshmem_offset[s]..
+    `shard_do_copy_mask` (int8, packing only) skips shards whose entry is 0.
+    """
+    if buffer is None:
+        raise RuntimeError("a2a_memcpy_non_cp: this build has no NVSHMEM dispatcher; pass buffer=")
+    _check_tensor(2, tensor, "tensor")
+    _check_tensor(1, nvshmem_offset, "seq_nvshmem_offset")
+    _check_dtype(nvshmem_offset, torch.int64, "seq_nvshmem_offset")
+    _check_dtype(shard_tokens, torch.int64, "seq_tokens")
+    num_seq = nvshmem_offset.size(0)
+    mask_ptr = None
+    if shard_do_copy_mask is not None:
+        _check_tensor(1, shard_do_copy_mask, "copy_seq_mask")
+        if shard_do_copy_mask.size(0) != num_seq:
+            raise RuntimeError("copy_seq_mask must be of shape (num_sequence,)")
+        _check_dtype(shard_do_copy_mask, torch.int8, "copy_seq_mask")
+        mask_ptr = shard_do_copy_mask.data_ptr()
+    if not buffer.is_cuda:
+        raise RuntimeError("tensor buffer must be on CUDA")
+    token_bytes = tensor.size(1) * tensor.element_size()
+    with torch.cuda.device(tensor.device):
+        rc = _lib.load().distca_memcpy_non_cp(
+            tensor.data_ptr(), buffer.data_ptr(), nvshmem_offset.data_ptr(), shard_tokens.data_ptr(),
+            mask_ptr, num_seq, token_bytes, tensor.size(0), 1 if to_nvshmem else 0, _stream())
+    _lib.check(rc, "a2a_memcpy_non_cp")
+    return None
+
+
+def a2a_memcpy_cp(
+    tensor: torch.Tensor, do_shard: torch.Tensor,
+    nvshmem_offset: torch.Tensor, shard_tokens: torch.Tensor,
+    to_nvshmem: bool, buffer: Optional[torch.Tensor] = None,
+    instance_id: Optional[int] = None,
+):
+    """Replicating pack of `tensor` [T, hidden] to every live (shard, replica) slot of
+    `buffer`, or unpack into `tensor` [max_cp, T, hidden] (which the caller pre-zeroes)."""
+    if buffer is None:
+        raise RuntimeError("a2a_memcpy_cp: this build has no NVSHMEM dispatcher; pass buffer=")
+    _check_tensor(2 if to_nvshmem else 3, tensor, "tensor")
+    if nvshmem_offset.dim() != 2:
+        raise RuntimeError("tensor seq_nvshmem_offset must have 2 dimensions")
+    num_seq = nvshmem_offset.size(1)
+    cp_degree = nvshmem_offset.size(0)
+    _check_tensor(1, shard_tokens, "seq_tokens")
+    if shard_tokens.size(0) != num_seq:
+        raise RuntimeError("seq_tokens must be of dimension (num_sequence)")
+    _check_tensor(2, do_shard, "do_shard")
+    if do_shard.size(0) != num_seq or do_shard.size(1) != cp_degree:
+        raise RuntimeError("do_shard must be of dimension (num_sequence, cp_degree)")
+    _check_dtype(do_shard, torch.int8, "do_shard")
+    _check_dtype(nvshmem_offset, torch.int64, "seq_nvshmem_offset")
+    _check_dtype(shard_tokens, torch.int64, "seq_tokens")
+    if not nvshmem_offset.is_contiguous():
+        raise RuntimeError("tensor seq_nvshmem_offset must be contiguous")
+    hidden_dim = 1 if to_nvshmem else 2
+    token_bytes = tensor.size(hidden_dim) * tensor.element_size()
+    num_tokens = tensor.size(0) if to_nvshmem else tensor.size(1)
+    with torch.cuda.device(tensor.device):
+        rc = _lib.load().distca_memcpy_cp(
+            tensor.data_ptr(), buffer.data_ptr(), do_shard.data_ptr(), nvshmem_offset.data_ptr(),
+            shard_tokens.data_ptr(), token_bytes, num_tokens, cp_degree, num_seq,
+            1 if to_nvshmem else 0, _stream())
+    _lib.check(rc, "a2a_memcpy_cp")
+    return None
+
+
+def pre_a2a_grad_acc(
+    tensor: torch.Tensor, num_copies: torch.Tensor,
+    copy_start_id: torch.Tensor, shard_tokens: torch.Tensor,
+):
+    """Sums the gradient rows of every duplicate KV copy into its main copy, in place, so
+    that only one gradient per shard has to be sent back."""
+    _check_tensor(2, tensor, "tensor")
+    _check_tensor(1, num_copies, "num_copies")
+    _check_tensor(1, shard_tokens, "seq_lens")
+    _check_tensor(2, copy_start_id, "copy_start_id")
+    num_seqs = num_copies.size(0)
+    if shard_tokens.size(0) != num_seqs:
+        raise RuntimeError("seq_lens must be of shape (num_sequence,)")
+    if copy_start_id.size(0) != num_seqs:
+        raise RuntimeError("copy_start_id must be of shape (num_sequence, max_num_copies)")
+    _check_dtype(num_copies, torch.int32, "num_copies")
+    _check_dtype(copy_start_id, torch.int64, "copy_start_id")
+    _check_dtype(shard_tokens, torch.int64, "seq_lens")
+    if tensor.dtype not in _DTYPE_CODE:
+        raise RuntimeError("Only fp32, fp16 and bf16 inputs are supported")
+    with torch.cuda.device(tensor.device):
+        rc = _lib.load().distca_grad_sum(
+            tensor.data_ptr(), _DTYPE_CODE[tensor.dtype], num_copies.data_ptr(), copy_start_id.data_ptr(),
+            shard_tokens.data_ptr(), tensor.size(0), tensor.size(1), num_seqs, copy_start_id.size(1), _stream())
+    _lib.check(rc, "pre_a2a_grad_acc")
+    return tensor

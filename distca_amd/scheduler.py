@@ -1,0 +1,51 @@
+"""Host mirror of the tile scheduler the attention kernels build on device.
+
+distca_ca_schedule_host runs the same cost functions and the same bin sort as the device
+builder, on host arrays, so the balance invariants can be checked without a GPU.  The
+reference has no GPU-side scheduler (flash-attn launches a static grid); the cost unit is
+the causal-pair count its planner balances across ranks (distca/planner/planner.py:366-378).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence, Tuple
+
+import numpy as np
+
+from . import _lib
+
+FWD, BWD = 0, 1
+
+
+def _params(cu_q, cu_k, hq, hkv, d, causal) -> _lib.CaParams:
+    cu_q = np.asarray(cu_q, dtype=np.int64)
+    cu_k = np.asarray(cu_k, dtype=np.int64)
+    lq, lk = np.diff(cu_q), np.diff(cu_k)
+    return _lib.CaParams(len(lq), int(cu_q[-1]), int(cu_k[-1]), hq, hkv, d,
+                         int(lq.max()) if len(lq) else 0, int(lk.max()) if len(lk) else 0,
+                         float(d) ** -0.5, 1 if causal else 0, 0, 0)
+
+
+def tile_shape(kind: int, hq: int, hkv: int, d: int = 128) -> Tuple[int, int]:
+    """(flattened query rows per block, keys per block) of the kernels of `kind`."""
+    p = _lib.CaParams(1, 1, 1, hq, hkv, d, 1, 1, 1.0, 1, 0, 0)
+    out = (ctypes.c_int32 * 2)()
+    _lib.check(_lib.load().distca_ca_tile_shape(kind, ctypes.byref(p), ctypes.byref(out)), "tile_shape")
+    return int(out[0]), int(out[1])
+
+
+def build_schedule(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequence[int], num_heads_q: int,
+                   num_heads_kv: int, head_dim: int = 128, causal: bool = True) -> np.ndarray:
+    """Work items as an int32 array [n, 3] of (task, block, cost), most expensive first."""
+    cu_q = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
+    cu_k = np.ascontiguousarray(cu_seqlens_k, dtype=np.int32)
+    p = _params(cu_q, cu_k, num_heads_q, num_heads_kv, head_dim, causal)
+    lib = _lib.load()
+    n = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), None, 0)
+    if n < 0:
+        _lib.check(int(n), "build_schedule")
+    items = np.zeros((int(n), 3), dtype=np.int32)
+    if n:
+        m = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), items.ctypes.data, int(n))
+        assert m == n
+    return items

@@ -1,0 +1,164 @@
+/*
+ * distca_ca.h — C ABI of the MI355X (gfx950) core-attention server library.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void* so the header needs no HIP include).  All work is enqueued
+ * asynchronously on `stream`; nothing synchronises with the host and nothing
+ * allocates device memory — scratch space is brought in by the caller as a
+ * workspace whose size the matching *_workspace_bytes() call reports.
+ *
+ * Return value: 0 on success, a negative DISTCA_E_* code on a rejected call.
+ * distca_last_error() returns a thread-local human readable message for the
+ * last non-zero return.
+ *
+ * Reference interfaces replaced (paths relative to the DistCA tree):
+ *   csrc/core/memcpy.h:5-47            launch_memcpy_non_cp / launch_memcpy_cp /
+ *                                      launch_inplace_grad_sum<T>
+ *   csrc/bindings/all_to_all.cpp:47-254 the torch-op wrappers around them
+ *   distca/runtime/megatron/ops/fused_comm_attn.py:151-197,259-272
+ *                                      the flash-attn varlen fwd / bwd invocation
+ */
+#ifndef DISTCA_CA_H_
+#define DISTCA_CA_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DISTCA_OK 0
+#define DISTCA_E_INVALID (-1)   /* bad argument (shape, alignment, null pointer)  */
+#define DISTCA_E_UNSUPPORTED (-2) /* valid request this build has no kernel for    */
+#define DISTCA_E_WORKSPACE (-3) /* workspace too small                             */
+#define DISTCA_E_LAUNCH (-4)    /* HIP reported an error at launch                 */
+
+/* element types of distca_grad_sum */
+#define DISTCA_DTYPE_F32 0
+#define DISTCA_DTYPE_F16 1
+#define DISTCA_DTYPE_BF16 2
+
+const char *distca_last_error(void);
+/* ABI version of this header: bumped whenever a signature changes. */
+int distca_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * fa2a shard pack / unpack.
+ *
+ * Replaces launch_memcpy_non_cp (csrc/core/memcpy.cu:240-282; kernel :22-74) as
+ * reached through fast_a2a_memcpy_non_cp[_debug] (csrc/bindings/all_to_all.cpp:
+ * 47-113).  `tensor` is a contiguous [num_tokens, token_bytes] byte matrix.
+ * Shard s owns rows [start_s, start_s + seq_tokens[s]) with start_s the
+ * exclusive prefix sum of seq_tokens, and the byte range
+ * [seq_offset[s], seq_offset[s] + seq_tokens[s]*token_bytes) of `buffer`.
+ * to_buffer != 0 packs tensor -> buffer, 0 unpacks buffer -> tensor.
+ * copy_seq_mask (int8 [num_seq], may be NULL) skips shards whose entry is 0;
+ * like the reference it is honoured only when packing.
+ * Rows at or beyond num_tokens are never touched.
+ * token_bytes, seq_offset[] and both base pointers must be multiples of 16.
+ * ------------------------------------------------------------------------- */
+int distca_memcpy_non_cp(void *tensor, void *buffer,
+                         const int64_t *seq_offset, const int64_t *seq_tokens,
+                         const int8_t *copy_seq_mask, int64_t num_seq,
+                         int64_t token_bytes, int64_t num_tokens, int to_buffer,
+                         void *stream);
+
+/* Replaces launch_memcpy_cp (csrc/core/memcpy.cu:285-343; kernel :77-155) as
+ * reached through fast_a2a_memcpy_cp[_debug] (all_to_all.cpp:116-179,243-254).
+ * Logical shard (c, s), c < max_cp, s < num_seq, is live iff
+ * do_shard[s*max_cp + c] != 0 and owns buffer bytes starting at
+ * seq_offset[c*num_seq + s].  Packing reads rows start_s.. of the
+ * [num_tokens, token_bytes] tensor for every live replica c; unpacking writes
+ * rows c*num_tokens + start_s.. of the [max_cp, num_tokens, token_bytes]
+ * tensor (which the caller pre-zeroes, dispatch_fn.py:79-80). */
+int distca_memcpy_cp(void *tensor, void *buffer, const int8_t *do_shard,
+                     const int64_t *seq_offset, const int64_t *seq_tokens,
+                     int64_t token_bytes, int64_t num_tokens, int32_t max_cp,
+                     int64_t num_seq, int to_buffer, void *stream);
+
+/* Replaces launch_inplace_grad_sum<T> (csrc/core/memcpy.cu:346-410; kernel
+ * :158-236) as reached through fast_a2a_grad_acc (all_to_all.cpp:182-240).
+ * For every shard s with num_copies[s] > 0 and every row t of it:
+ *   data[start_s + t] += data[copy_start_id[s*max_copies + c] + t],
+ * c = 0 .. num_copies[s]-1 in that order, each addition rounded to `dtype`. */
+int distca_grad_sum(void *data, int dtype, const int32_t *num_copies,
+                    const int64_t *copy_start_id, const int64_t *seq_lens,
+                    int64_t num_tokens, int64_t hidden, int64_t num_seq,
+                    int64_t max_copies, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Core attention over a batch of CA tasks.
+ *
+ * Task b: query rows q[cu_seqlens_q[b] .. cu_seqlens_q[b+1]) (Lq rows) attend
+ * to key/value rows k[ks .. ks+Lk) with Lk = cu_seqlens_k[b+1]-cu_seqlens_k[b]
+ * and ks = kv_task_offsets ? kv_task_offsets[b] : cu_seqlens_k[b].  With
+ * causal != 0 row i sees column j iff j <= i + (Lk - Lq) (bottom-right
+ * aligned, the flash-attn 2.1+ convention the reference relies on at
+ * per_doc_cp_attn.py:326,406-411).  q-head h reads kv-head h / (Hq/Hkv).
+ *
+ * Layouts: q,out,dout,dq [total_q, Hq, D] bf16; k,v,dk,dv [total_k, Hkv, D]
+ * bf16; lse [Hq, total_q] fp32 natural-log with the scale included;
+ * cu_seqlens_* int32 [B+1]; kv_task_offsets int32 [B] or NULL.
+ * D must be 128 in this build.
+ *
+ * These two calls stand where fused_comm_attn.py:151-197 calls
+ * flash_attn's varlen forward and :259-272 its varlen backward.
+ * ------------------------------------------------------------------------- */
+typedef struct distca_ca_params {
+  int32_t num_tasks;    /* B                                                  */
+  int32_t total_q;      /* rows of q / out                                    */
+  int32_t total_k;      /* rows of k / v                                      */
+  int32_t num_heads_q;  /* Hq                                                 */
+  int32_t num_heads_kv; /* Hkv, divides Hq                                    */
+  int32_t head_dim;     /* D                                                  */
+  int32_t max_seqlen_q; /* upper bound of any task's Lq                       */
+  int32_t max_seqlen_k; /* upper bound of any task's Lk                       */
+  float softmax_scale;  /* multiplies q.k before softmax                      */
+  int32_t causal;       /* 0 / 1                                              */
+  int32_t deterministic;/* backward only: 1 = no floating-point atomics       */
+  int32_t reserved;
+} distca_ca_params;
+
+int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p);
+int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p);
+
+int distca_ca_fwd(const void *q, const void *k, const void *v, void *out,
+                  float *lse, const int32_t *cu_seqlens_q,
+                  const int32_t *cu_seqlens_k, const int32_t *kv_task_offsets,
+                  const distca_ca_params *p, void *workspace,
+                  int64_t workspace_bytes, void *stream);
+
+/* dk/dv rows are written once per task when kv_task_offsets is NULL.  When it
+ * is given, tasks may alias KV rows and dk/dv hold the sum over every task
+ * that read the row (what the reference obtains with duplicated KV copies and
+ * inplace_grad_sum_kernel). */
+int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v,
+                  const void *out, const float *lse, void *dq, void *dk,
+                  void *dv, const int32_t *cu_seqlens_q,
+                  const int32_t *cu_seqlens_k, const int32_t *kv_task_offsets,
+                  const distca_ca_params *p, void *workspace,
+                  int64_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Tile scheduler, host mirror.  The device builds the same list inside
+ * distca_ca_fwd / distca_ca_bwd; this entry point runs the identical code on
+ * host arrays so the balance invariants can be tested without a GPU.
+ * kind 0 = forward (one item per (task, block of query rows), cost = KV tiles
+ * visible to the block), 1 = backward (one item per (task, KV block), cost =
+ * query blocks that see it).  Writes up to max_items (task, block, cost)
+ * triples sorted by descending cost and returns the item count, or a negative
+ * error.  The reference has no counterpart: flash-attn launches a static
+ * (m-block, batch, head) grid sized by max_seqlen_q.
+ * ------------------------------------------------------------------------- */
+int64_t distca_ca_schedule_host(int kind, const int32_t *cu_seqlens_q,
+                                const int32_t *cu_seqlens_k,
+                                const distca_ca_params *p, int32_t *items,
+                                int64_t max_items);
+/* tile geometry used by the kernels of `kind` for the head layout in p:
+ * out[0] = query rows (tokens) per block, out[1] = kv rows per block. */
+int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DISTCA_CA_H_ */

@@ -1,0 +1,79 @@
+"""GPU parity of the HIP attention kernels (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close_bf16, cu, make_qkv
+from oracle.attention import ca_reference_bwd, ca_reference_fwd
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128):
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    cu_q, cu_k = cu(q_lens), cu(k_lens)
+    tq = int(cu_q[-1])
+    tk = int(total_k if total_k is not None else cu_k[-1])
+    q, k, v, do = make_qkv(tq, tk, hq, hkv, d, seed)
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_q, cu_k, causal=causal, kv_task_offsets=kv_offsets)
+    dcu_q = torch.tensor(cu_q, device=cuda)
+    dcu_k = torch.tensor(cu_k, device=cuda)
+    dkv = torch.tensor(np.asarray(kv_offsets, dtype=np.int32), device=cuda) if kv_offsets is not None else None
+    qd, kd, vd, dod = q.to(cuda), k.to(cuda), v.to(cuda), do.to(cuda)
+    print(f"case q_lens={list(q_lens)[:6]} k_lens={list(k_lens)[:6]} hq={hq} hkv={hkv} causal={causal} alias={kv_offsets is not None}", flush=True)
+    out, lse = ca_varlen_fwd(qd, kd, vd, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal, dkv)
+    torch.cuda.synchronize()
+    assert_close_bf16(out, ref_out, "out")
+    finite = torch.isfinite(ref_lse)
+    lse_c = lse.cpu()
+    assert torch.equal(torch.isfinite(lse_c), finite)
+    assert (lse_c[finite] - ref_lse[finite]).abs().max().item() <= 2e-3, "lse"
+    if not bwd:
+        return
+    # the oracle consumes the same (out, lse) the kernel is handed, as the reference's backward does
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_q, cu_k, causal=causal, kv_task_offsets=kv_offsets,
+                                              out=out.cpu(), softmax_lse=lse.cpu())
+    dq, dk, dv = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal,
+                               False, dkv)
+    torch.cuda.synchronize()
+    assert_close_bf16(dq, ref_dq, "dq")
+    assert_close_bf16(dk, ref_dk, "dk")
+    assert_close_bf16(dv, ref_dv, "dv")
+
+
+def test_config1_tiny_forward(cuda):
+    """BASELINE config 1: docs [512, 1024, 2560], 32q/8kv, d128, causal, forward."""
+    _run([512, 1024, 2560], [512, 1024, 2560], 32, 8, 1, cuda, bwd=False)
+
+
+@pytest.mark.parametrize("lens", [[64], [1], [33, 1, 130], [257, 255, 256, 3]])
+def test_whole_docs_fwd_bwd_small(cuda, lens):
+    _run(lens, lens, 8, 2, 7, cuda)
+
+
+def test_whole_docs_fwd_bwd_medium(cuda):
+    _run([512, 1024, 700], [512, 1024, 700], 32, 8, 2, cuda)
+
+
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 1), (6, 2), (16, 2)])
+def test_head_groupings(cuda, hq, hkv):
+    """MHA, MQA, a non-power-of-two group and the Llama-3-70B group of 8."""
+    _run([300, 45], [300, 45], hq, hkv, 3, cuda)
+
+
+def test_prefix_tasks_lk_gt_lq(cuda):
+    """CA tasks: query shard shorter than its KV prefix (bottom-right causal)."""
+    _run([128, 200, 64], [384, 200, 1000], 8, 2, 4, cuda)
+
+
+def test_shared_kv_prefix(cuda):
+    """Three shards of one 600-token document reading one stored KV copy."""
+    _run([200, 150, 250], [200, 350, 600], 8, 2, 5, cuda, kv_offsets=[0, 0, 0], total_k=600)
+
+
+def test_non_causal(cuda):
+    _run([100, 260], [100, 260], 4, 2, 6, cuda, causal=False)
+
+
+def test_empty_task(cuda):
+    _run([128, 0, 70], [128, 0, 70], 4, 2, 8, cuda)

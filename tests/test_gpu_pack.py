@@ -1,0 +1,125 @@
+"""GPU parity (bit-exact) of the shard pack / unpack / grad-sum kernels against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fa2a
+
+pytestmark = pytest.mark.gpu
+
+
+def _layout(rng, lens, token_bytes, slack=64):
+    perm = rng.permutation(len(lens))
+    off = np.zeros(len(lens), dtype=np.int64)
+    cur = 16 * int(rng.integers(0, 4))
+    for s in perm:
+        off[s] = cur
+        cur += int(lens[s]) * token_bytes + 16 * int(rng.integers(0, slack))
+    return off, cur
+
+
+@pytest.mark.parametrize("hidden,dtype", [(128, torch.bfloat16), (1024, torch.bfloat16), (4096, torch.bfloat16), (24, torch.float32), (8320, torch.uint8)])
+@pytest.mark.parametrize("nshard", [1, 7, 300])
+def test_non_cp_pack_unpack(cuda, hidden, dtype, nshard):
+    from distca_amd.ops import a2a_memcpy_non_cp
+    rng = np.random.default_rng(hidden * 1000 + nshard)
+    lens = rng.integers(0, 40, size=nshard).astype(np.int64)
+    lens[rng.integers(0, nshard)] += 5
+    T = int(lens.sum())
+    esz = torch.empty((), dtype=dtype).element_size()
+    tb = hidden * esz
+    off, nbuf = _layout(rng, lens, tb)
+    src = torch.from_numpy(rng.integers(0, 256, size=(T, tb), dtype=np.uint8)).view(dtype).reshape(T, hidden)
+    mask = (rng.random(nshard) < 0.7).astype(np.int8)
+    for use_mask in (False, True):
+        buf0 = rng.integers(0, 256, size=nbuf, dtype=np.uint8)
+        exp = buf0.copy()
+        fa2a.copy_non_cp(src.view(torch.uint8).numpy().reshape(T, tb), exp, off, lens, mask if use_mask else None, True)
+        dbuf = torch.from_numpy(buf0.copy()).to(cuda)
+        print(f"pack hidden={hidden} {dtype} nshard={nshard} mask={use_mask}", flush=True)
+        a2a_memcpy_non_cp(src.to(cuda), torch.from_numpy(off).to(cuda), torch.from_numpy(lens).to(cuda), True,
+                          torch.from_numpy(mask).to(cuda) if use_mask else None, buffer=dbuf)
+        torch.cuda.synchronize()
+        assert np.array_equal(dbuf.cpu().numpy(), exp)
+    # unpack the unmasked pack into a poisoned tensor: identity
+    dst = torch.full((T, tb), 0xA5, dtype=torch.uint8, device=cuda).view(dtype).reshape(T, hidden)
+    a2a_memcpy_non_cp(dst, torch.from_numpy(off).to(cuda), torch.from_numpy(lens).to(cuda), False, None, buffer=dbuf if not use_mask else torch.from_numpy(exp).to(cuda))
+    exp_t = np.full((T, tb), 0xA5, dtype=np.uint8)
+    fa2a.copy_non_cp(exp_t, exp, off, lens, None, False)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.view(torch.uint8).reshape(T, tb).cpu().numpy(), exp_t)
+
+
+@pytest.mark.parametrize("max_cp", [1, 3])
+def test_cp_pack_unpack(cuda, max_cp):
+    from distca_amd.ops import a2a_memcpy_cp
+    rng = np.random.default_rng(77 + max_cp)
+    nshard, hidden = 9, 1024
+    lens = rng.integers(1, 50, size=nshard).astype(np.int64)
+    T = int(lens.sum())
+    tb = hidden * 2
+    do_shard = (rng.random((nshard, max_cp)) < 0.6).astype(np.int8)
+    do_shard[:, 0] = 1
+    off = np.zeros((max_cp, nshard), dtype=np.int64)
+    cur = 0
+    for c in range(max_cp):
+        for s in rng.permutation(nshard):
+            off[c, s] = cur
+            cur += int(lens[s]) * tb
+    src = torch.from_numpy(rng.integers(0, 256, size=(T, tb), dtype=np.uint8))
+    exp = np.zeros(cur, dtype=np.uint8)
+    fa2a.copy_cp(src.numpy(), exp, do_shard, off, lens, True)
+    dbuf = torch.zeros(cur, dtype=torch.uint8, device=cuda)
+    d_do, d_off, d_len = (torch.from_numpy(x).to(cuda) for x in (do_shard, off, lens))
+    print(f"cp pack max_cp={max_cp}", flush=True)
+    a2a_memcpy_cp(src.view(torch.bfloat16).to(cuda), d_do, d_off, d_len, True, buffer=dbuf)
+    torch.cuda.synchronize()
+    assert np.array_equal(dbuf.cpu().numpy(), exp)
+    planes = torch.zeros((max_cp, T, hidden), dtype=torch.bfloat16, device=cuda)
+    a2a_memcpy_cp(planes, d_do, d_off, d_len, False, buffer=dbuf)
+    exp_p = np.zeros((max_cp, T, tb), dtype=np.uint8)
+    fa2a.copy_cp(exp_p, exp, do_shard, off, lens, False)
+    torch.cuda.synchronize()
+    assert np.array_equal(planes.view(torch.uint8).reshape(max_cp, T, tb).cpu().numpy(), exp_p)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("hidden", [128, 1024, 20])
+def test_grad_sum(cuda, dtype, hidden):
+    from distca_amd.ops import pre_a2a_grad_acc
+    rng = np.random.default_rng(hidden)
+    # shards: mains with copies interleaved with plain shards
+    lens, num_copies, starts = [], [], []
+    spec = [(37, 2), (5, 0), (64, 1), (1, 3), (12, 0)]
+    order = []
+    for i, (ln, nc) in enumerate(spec):
+        order.append((i, ln, nc, True))
+        for c in range(nc):
+            order.append((i, ln, 0, False))
+    perm = rng.permutation(len(order))
+    order = [order[i] for i in perm]
+    pos, main_idx, copy_pos = 0, {}, {}
+    for j, (i, ln, nc, is_main) in enumerate(order):
+        if is_main:
+            main_idx[i] = j
+        else:
+            copy_pos.setdefault(i, []).append(pos)
+        lens.append(ln)
+        pos += ln
+    T = pos
+    max_copies = 3
+    nc_arr = np.zeros(len(order), dtype=np.int32)
+    cs = np.zeros((len(order), max_copies), dtype=np.int64)
+    for i, (ln, nc) in enumerate(spec):
+        nc_arr[main_idx[i]] = nc
+        for c, p in enumerate(copy_pos.get(i, [])):
+            cs[main_idx[i], c] = p
+    g = torch.Generator().manual_seed(hidden)
+    data = (torch.randn((T, hidden), generator=g) * 3).to(dtype)
+    exp = data.clone()
+    fa2a.grad_sum(exp, nc_arr, cs, lens)
+    d = data.to(cuda)
+    print(f"grad_sum {dtype} hidden={hidden}", flush=True)
+    pre_a2a_grad_acc(d, torch.from_numpy(nc_arr).to(cuda), torch.from_numpy(cs).to(cuda), torch.tensor(lens, dtype=torch.int64, device=cuda))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().view(torch.uint8), exp.view(torch.uint8))
