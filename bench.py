@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the CA-server hot path on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input: varlen causal
+attention forward + backward over the CA-task batch of the benchmark configuration
+"Llama-3-8B heads, 131 072 packed tokens" (32 q heads / 8 kv heads, head_dim 128, bf16,
+document lengths lognormal(8, 1.5) clipped to [128, 65 536]).  Inputs are resident in HBM
+before the timed region.  One JSON line is printed on stdout; a human-readable table goes
+to stderr.
+
+Algorithmic work: causal pairs P = sum_tasks [Lq*Lk - Lq(Lq-1)/2]; forward 4*Hq*D*P FLOP,
+backward 10*Hq*D*P FLOP.  `roofline` describes the dominant kernel (the attention backward
+kernel) with its launch duration measured live by HIP events the library records on the
+launch stream.  `cpu_baseline` times the CPU oracle (per-document fp32 PyTorch attention,
+forward + backward) on this box's host cores over a bounded sample of the same documents.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(batch, budget_s: float, seed: int):
+    """Oracle forward+backward on host cores over the shortest documents of the batch until
+    about `budget_s` seconds have been spent; TFLOP/s over the FLOPs actually executed."""
+    import torch
+    from oracle.attention import ca_reference_bwd, ca_reference_fwd, causal_pairs
+    hq, hkv, d = batch.num_heads_q, batch.num_heads_kv, batch.head_dim
+    order = np.argsort(batch.q_lens, kind="stable")
+    g = torch.Generator().manual_seed(seed)
+    spent, flops, docs, tokens = 0.0, 0, 0, 0
+    for b in order:
+        n = int(batch.q_lens[b])
+        if n > 8192:
+            break
+        q = torch.randn((n, hq, d), generator=g).to(torch.bfloat16)
+        k = torch.randn((n, hkv, d), generator=g).to(torch.bfloat16)
+        v = torch.randn((n, hkv, d), generator=g).to(torch.bfloat16)
+        do = torch.randn((n, hq, d), generator=g).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        ca_reference_fwd(q, k, v, [0, n], [0, n])
+        ca_reference_bwd(do, q, k, v, [0, n], [0, n])
+        spent += time.perf_counter() - t0
+        flops += 14 * hq * d * causal_pairs(n, n)
+        docs += 1
+        tokens += n
+        if spent >= budget_s:
+            break
+    return {
+        "value": round(flops / max(spent, 1e-9) / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle fwd+bwd (fp32 PyTorch, per document) on the {docs} shortest documents of the workload "
+                  f"({tokens} tokens, {flops:.3e} FLOP) in {spent:.1f} s",
+    }
+
+
+def pack_unpack_bench(torch, dev, iters: int = 10):
+    """fa2a pack / unpack of 262 144 tokens of q (8 192 B) + k, v (2 048 B each): GB/s over
+    algorithmic bytes (read + write of the payload)."""
+    from distca_amd import _lib
+    from distca_amd.ops import a2a_memcpy_non_cp
+    from distca_amd.workloads import config4_pack
+    lay = config4_pack()
+    T = lay.num_tokens
+    tens = {n: torch.randint(-32768, 32767, (T, tb // 2), dtype=torch.int16, device=dev).view(torch.bfloat16)
+            for n, tb in lay.token_bytes.items()}
+    buf = torch.empty(lay.buffer_bytes, dtype=torch.uint8, device=dev)
+    lens = torch.from_numpy(lay.seq_tokens).to(dev)
+    offs = {n: torch.from_numpy(o).to(dev) for n, o in lay.offsets.items()}
+    payload = sum(T * tb for tb in lay.token_bytes.values())
+    res = {}
+    for direction, to_buf in (("pack", True), ("unpack", False)):
+        for _ in range(2):
+            for n in tens:
+                a2a_memcpy_non_cp(tens[n], offs[n], lens, to_buf, buffer=buf)
+        torch.cuda.synchronize()
+        _lib.timing_read(_lib.TIMER_MEMCPY_NON_CP)
+        _lib.timing_enable(True)
+        for _ in range(iters):
+            for n in tens:
+                a2a_memcpy_non_cp(tens[n], offs[n], lens, to_buf, buffer=buf)
+        torch.cuda.synchronize()
+        _lib.timing_enable(False)
+        ms, launches = _lib.timing_read(_lib.TIMER_MEMCPY_NON_CP)
+        gbps = 2 * payload * iters / (ms * 1e-3) / 1e9
+        res[direction] = {"GB/s": round(gbps, 1), "frac_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
+                          "ms_per_pass": round(ms / iters, 4), "launches": launches}
+    res["workload"] = f"{lay.name}: {len(lay.seq_tokens)} shards, payload {payload} B per direction"
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU-baseline leg (0 disables)")
+    ap.add_argument("--tokens", type=int, default=131072)
+    ap.add_argument("--no-pack", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the CA-server path; --gpus must be 1 "
+                 "(this build has no multi-GPU transport)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from distca_amd import _lib
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    from distca_amd.workloads import config2_llama8b_128k
+    _lib.load()
+    dev = torch.device("cuda:0")
+    batch = config2_llama8b_128k(total=args.tokens)
+    hq, hkv, d = batch.num_heads_q, batch.num_heads_kv, batch.head_dim
+    tq = batch.total_q
+    flop_fwd, flop_bwd = batch.flops()
+    log(f"workload {batch.name}: {len(batch.q_lens)} docs, max {int(batch.q_lens.max())}, causal pairs {batch.causal_pairs:.4e}, "
+        f"fwd {flop_fwd:.4e} FLOP, bwd {flop_bwd:.4e} FLOP")
+
+    gen = torch.Generator(device=dev).manual_seed(1002)
+    q = torch.randn((tq, hq, d), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    k = torch.randn((tq, hkv, d), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    v = torch.randn((tq, hkv, d), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    do = torch.randn((tq, hq, d), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    cu_q = torch.from_numpy(batch.cu_seqlens_q).to(dev)
+    cu_k = torch.from_numpy(batch.cu_seqlens_k).to(dev)
+    max_q, max_k = int(batch.q_lens.max()), int(batch.k_lens.max())
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+    def step():
+        out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, max_q, max_k, None, True)
+        ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, max_q, max_k, None, True, False, None, dq, dk, dv)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    for t in (_lib.TIMER_CA_FWD, _lib.TIMER_CA_BWD):
+        _lib.timing_read(t)
+    _lib.timing_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    _lib.timing_enable(False)
+    fwd_ms, fwd_n = _lib.timing_read(_lib.TIMER_CA_FWD)
+    bwd_ms, bwd_n = _lib.timing_read(_lib.TIMER_CA_BWD)
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    tflops = (flop_fwd + flop_bwd) / (ms_per_step * 1e-3) / 1e12
+    fwd_k = fwd_ms / max(fwd_n, 1)
+    bwd_k = bwd_ms / max(bwd_n, 1)
+    fwd_tf = flop_fwd / (fwd_k * 1e-3) / 1e12
+    bwd_tf = flop_bwd / (bwd_k * 1e-3) / 1e12
+    log(f"step {ms_per_step:.3f} ms  -> {tflops:.1f} TFLOP/s fwd+bwd ({100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak)")
+    log(f"  ca_fwd_kernel {fwd_k:.3f} ms -> {fwd_tf:.1f} TFLOP/s ({100 * fwd_tf / PEAK_BF16_TFLOPS:.1f}%)")
+    log(f"  ca_bwd_kernel {bwd_k:.3f} ms -> {bwd_tf:.1f} TFLOP/s ({100 * bwd_tf / PEAK_BF16_TFLOPS:.1f}%)")
+
+    pack = None
+    if not args.no_pack:
+        del dq, dk, dv
+        pack = pack_unpack_bench(torch, dev)
+        log(f"  pack   {pack['pack']['GB/s']} GB/s ({100 * pack['pack']['frac_hbm_peak']:.1f}% of HBM peak)")
+        log(f"  unpack {pack['unpack']['GB/s']} GB/s ({100 * pack['unpack']['frac_hbm_peak']:.1f}% of HBM peak)")
+
+    cpu = None
+    if args.cpu_seconds > 0:
+        cpu = cpu_baseline(batch, args.cpu_seconds, 77)
+        log(f"  cpu baseline {cpu['value']} TFLOP/s on {cpu['cores']} threads: {cpu['sample']}")
+
+    line = {
+        "metric": "causal-attn TFLOP/s fwd+bwd, Llama-3-8B heads, 128K varlen; % MFMA peak",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{batch.name}: {len(batch.q_lens)} whole documents, lognormal(8,1.5) lengths in [128,65536], "
+                               f"{tq} packed tokens, 32q/8kv heads, d=128, causal, fwd+bwd",
+                   "causal_pairs": batch.causal_pairs, "flop_fwd": flop_fwd, "flop_bwd": flop_bwd,
+                   "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2)},
+        "roofline": {"bound": "mfma", "kernel": "ca_bwd_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(bwd_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "avg_launch_ms": round(bwd_k, 4), "launches": bwd_n,
+                     "also": {"ca_fwd_kernel": {"achieved": round(fwd_tf, 2), "frac": round(fwd_tf / PEAK_BF16_TFLOPS, 4),
+                                                "avg_launch_ms": round(fwd_k, 4), "launches": fwd_n}}},
+        "cpu_baseline": cpu,
+        "pack_unpack": pack,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

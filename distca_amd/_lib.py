@@ -40,6 +40,8 @@ SYMBOLS = {
                               POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_schedule_host": (c_int64, [c_int, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64]),
+    "distca_timing_enable": (None, [c_int]),
+    "distca_timing_read": (c_int, [c_int, POINTER(ctypes.c_double), POINTER(c_int64)]),
     "distca_ca_tile_shape": (c_int, [c_int, POINTER(CaParams), POINTER(c_int32 * 2)]),
 }
 
@@ -64,6 +66,20 @@ def load() -> ctypes.CDLL:
         raise RuntimeError(f"libdistca_ca.so ABI {lib.distca_abi_version()} != binding ABI {ABI_VERSION}: rebuild")
     _lib = lib
     return lib
+
+
+TIMER_CA_FWD, TIMER_CA_BWD, TIMER_MEMCPY_NON_CP, TIMER_MEMCPY_CP, TIMER_GRAD_SUM = range(5)
+
+
+def timing_enable(on: bool) -> None:
+    load().distca_timing_enable(1 if on else 0)
+
+
+def timing_read(which: int):
+    """(total milliseconds, launches) of kernel `which` since the last read."""
+    ms, n = ctypes.c_double(0), c_int64(0)
+    check(load().distca_timing_read(which, ctypes.byref(ms), ctypes.byref(n)), "timing_read")
+    return ms.value, n.value
 
 
 def check(rc: int, what: str) -> None:

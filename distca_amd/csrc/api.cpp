@@ -1,6 +1,9 @@
 // Process-wide state behind the C ABI: error text and device facts.
 #include "api_util.h"
 
+#include <utility>
+#include <vector>
+
 namespace distca {
 
 char *error_buffer() {
@@ -20,7 +23,61 @@ int num_compute_units() {
   return cached[dev];
 }
 
+namespace {
+struct TimerState {
+  bool enabled = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> pending[DISTCA_TIMER_COUNT];
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> pool;
+};
+TimerState &timers() {
+  static TimerState t;
+  return t;
+}
+}  // namespace
+
+void timer_begin(int which, hipStream_t stream) {
+  TimerState &t = timers();
+  if (!t.enabled || which < 0 || which >= DISTCA_TIMER_COUNT) return;
+  std::pair<hipEvent_t, hipEvent_t> ev;
+  if (!t.pool.empty()) {
+    ev = t.pool.back();
+    t.pool.pop_back();
+  } else if (hipEventCreate(&ev.first) != hipSuccess || hipEventCreate(&ev.second) != hipSuccess) {
+    return;
+  }
+  (void)hipEventRecord(ev.first, stream);
+  t.pending[which].push_back(ev);
+}
+
+void timer_end(int which, hipStream_t stream) {
+  TimerState &t = timers();
+  if (!t.enabled || which < 0 || which >= DISTCA_TIMER_COUNT || t.pending[which].empty()) return;
+  (void)hipEventRecord(t.pending[which].back().second, stream);
+}
+
 }  // namespace distca
+
+extern "C" void distca_timing_enable(int on) { distca::timers().enabled = on != 0; }
+
+extern "C" int distca_timing_read(int which, double *total_ms, int64_t *launches) {
+  using namespace distca;
+  if (which < 0 || which >= DISTCA_TIMER_COUNT || !total_ms || !launches) return fail(DISTCA_E_INVALID, "timing_read: bad argument");
+  TimerState &t = timers();
+  double sum = 0;
+  int64_t n = 0;
+  for (auto &ev : t.pending[which]) {
+    float ms = 0.f;
+    if (hipEventSynchronize(ev.second) == hipSuccess && hipEventElapsedTime(&ms, ev.first, ev.second) == hipSuccess) {
+      sum += ms;
+      ++n;
+    }
+    t.pool.push_back(ev);
+  }
+  t.pending[which].clear();
+  *total_ms = sum;
+  *launches = n;
+  return DISTCA_OK;
+}
 
 extern "C" const char *distca_last_error(void) { return distca::error_buffer(); }
 extern "C" int distca_abi_version(void) { return 1; }

@@ -27,6 +27,16 @@ inline int check_launch(const char *what) {
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Brackets a kernel launch with events when timing is enabled (see distca_timing_enable).
+void timer_begin(int which, hipStream_t stream);
+void timer_end(int which, hipStream_t stream);
+struct ScopedTimer {
+  int which;
+  hipStream_t stream;
+  ScopedTimer(int w, hipStream_t s) : which(w), stream(s) { timer_begin(w, s); }
+  ~ScopedTimer() { timer_end(which, stream); }
+};
+
 // Number of compute units of the current device (cached per device id).
 int num_compute_units();
 

@@ -503,10 +503,13 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
     if (e1 != hipSuccess || e2 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS", L::kTotal);
     attr_set = true;
   }
-  if (alias)
-    hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, true>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
-  else
-    hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, false>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
+  {
+    ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
+    if (alias)
+      hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, true>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
+    else
+      hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, false>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
+  }
 
   hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(q_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dq_acc), (__bf16 *)dq, q_elems / 8);
   if (alias) {

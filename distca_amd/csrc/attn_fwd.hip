@@ -342,6 +342,9 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
     if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
     attr_set = true;
   }
-  hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kFwdLds, s, a);
+  {
+    ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);
+    hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kFwdLds, s, a);
+  }
   return check_launch("ca_fwd");
 }

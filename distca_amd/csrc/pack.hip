@@ -278,6 +278,7 @@ extern "C" int distca_memcpy_non_cp(void *tensor, void *buffer, const int64_t *s
   int64_t per = slice_tokens(num_tokens, token_bytes, &grid);
   hipStream_t s = (hipStream_t)stream;
   uint8_t *t = (uint8_t *)tensor, *b = (uint8_t *)buffer;
+  ScopedTimer timer(DISTCA_TIMER_MEMCPY_NON_CP, s);
   if (to_buffer)
     hipLaunchKernelGGL((pack_kernel<true, false>), dim3(grid), dim3(kPackThreads), 0, s, t, b, seq_offset, seq_tokens,
                        copy_seq_mask, num_seq, token_bytes, num_tokens, 1, per);
@@ -300,6 +301,7 @@ extern "C" int distca_memcpy_cp(void *tensor, void *buffer, const int8_t *do_sha
   int64_t per = slice_tokens(num_tokens * max_cp, token_bytes, &grid);
   hipStream_t s = (hipStream_t)stream;
   uint8_t *t = (uint8_t *)tensor, *b = (uint8_t *)buffer;
+  ScopedTimer timer(DISTCA_TIMER_MEMCPY_CP, s);
   if (to_buffer)
     hipLaunchKernelGGL((pack_kernel<true, true>), dim3(grid), dim3(kPackThreads), 0, s, t, b, seq_offset, seq_tokens, do_shard,
                        num_seq, token_bytes, num_tokens, max_cp, per);
@@ -320,6 +322,7 @@ extern "C" int distca_grad_sum(void *data, int dtype, const int32_t *num_copies,
   int grid;
   int64_t per = slice_tokens(num_tokens, hidden * esz, &grid);
   hipStream_t s = (hipStream_t)stream;
+  ScopedTimer timer(DISTCA_TIMER_GRAD_SUM, s);
   switch (dtype) {
     case DISTCA_DTYPE_F32:
       hipLaunchKernelGGL((grad_sum_kernel<float>), dim3(grid), dim3(kPackThreads), 0, s, (float *)data, num_copies,

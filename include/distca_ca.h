@@ -158,6 +158,24 @@ int64_t distca_ca_schedule_host(int kind, const int32_t *cu_seqlens_q,
  * out[0] = query rows (tokens) per block, out[1] = kv rows per block. */
 int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
 
+/* ---------------------------------------------------------------------------
+ * Per-kernel timing, for benchmarks.  No counterpart in the reference (which
+ * wraps CUDA events around its flash-attn calls in Python,
+ * tests/test_e2e_combined.py:1947-1999).  While enabled, every entry point
+ * brackets its dominant kernel with HIP events recorded on the stream the
+ * kernel is launched on; distca_timing_read waits for those events, returns
+ * the summed duration and launch count of kernel `which` since the last read
+ * and clears them.  Not thread safe; leave disabled outside benchmarks.
+ * ------------------------------------------------------------------------- */
+#define DISTCA_TIMER_CA_FWD 0      /* ca_fwd_kernel                          */
+#define DISTCA_TIMER_CA_BWD 1      /* ca_bwd_kernel                          */
+#define DISTCA_TIMER_MEMCPY_NON_CP 2
+#define DISTCA_TIMER_MEMCPY_CP 3
+#define DISTCA_TIMER_GRAD_SUM 4
+#define DISTCA_TIMER_COUNT 5
+void distca_timing_enable(int on);
+int distca_timing_read(int which, double *total_ms, int64_t *launches);
+
 #ifdef __cplusplus
 }
 #endif
