@@ -20,6 +20,10 @@ HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-x", "hip",
     # scalar fp32 only: keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # select MFMAs with VGPR accumulators; the allocator moves long-lived ones to AGPRs itself.
+    # (AGPR-form selection, the default above 256 registers, copies every accumulator the VALU
+    # touches between the two files each loop iteration.)
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
 ]
 
@@ -42,23 +46,32 @@ def _compile(src: str, obj: str, extra: list[str]) -> None:
         sys.stderr.write(err + "\n")
 
 
-def build_library(extra_flags: list[str] | None = None, verbose: bool = False) -> str:
+def build_library(extra_flags: list[str] | None = None, verbose: bool = False, out_path: str | None = None) -> str:
+    """Compiles and links; `out_path` (default distca_amd/libdistca_ca.so) lets a tuning run
+    keep several variants side by side (select one with DISTCA_LIB_PATH)."""
     extra = list(extra_flags or [])
-    obj_dir = os.path.join(PKG_DIR, "build")
+    lib_path = out_path or LIB_PATH
+    obj_dir = os.path.join(PKG_DIR, "build", os.path.basename(lib_path))
     os.makedirs(obj_dir, exist_ok=True)
     objs = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), 6)) as ex:
         list(ex.map(lambda so: _compile(so[0], so[1], extra), zip(SOURCES, objs)))
-    tmp = LIB_PATH + ".tmp"
+    tmp = lib_path + ".tmp"
     cmd = [_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
     if verbose:
-        print("built", LIB_PATH)
-    return LIB_PATH
+        print("built", lib_path)
+    return lib_path
 
 
 if __name__ == "__main__":
-    build_library(sys.argv[1:], verbose=True)
+    argv = sys.argv[1:]
+    out = None
+    if "-o" in argv:
+        i = argv.index("-o")
+        out = os.path.abspath(argv[i + 1])
+        del argv[i:i + 2]
+    build_library(argv, verbose=True, out_path=out)

@@ -3,20 +3,25 @@
 // Stands where the reference calls flash-attn's varlen backward
 // (distca/runtime/megatron/ops/fused_comm_attn.py:259-272).
 //
-// Three launches on the caller's stream:
-//   1. bwd_prepare:  delta[h][t] = <dO, O> per (token, head), and zero the fp32 dQ accumulator.
-//   2. ca_bwd_kernel: one workgroup per (task, block of kBwdKV keys, kv head), in the order
-//      of the tile schedule.  Each wave keeps K and V of its 32*KSUB keys as MFMA B operands in
-//      registers together with the fp32 dK^T / dV^T accumulators, and the workgroup streams
-//      the query side (Q, dO, LSE, delta of every head of the group, flattened like the
-//      forward) through LDS in blocks of 32*MSUB rows, starting at the first block the causal
-//      mask lets see these keys.  Per block: S = Q K^T and dP = dO V^T (A from LDS, B from
-//      registers); P = exp2(S*c - LSE), dS = P (dP - delta) * scale in registers;
-//      dV^T += dO^T P and dK^T += Q^T dS with the A operand fetched by transposing LDS reads
-//      of the same row-major tiles and the B operand being the accumulator registers
-//      converted to bf16 in place; dS goes through LDS once so that each wave can form a
-//      32-column slice of dQ = dS K over all keys of the workgroup, which is added to the
-//      fp32 accumulator with hardware float atomics.
+// Launches on the caller's stream:
+//   1. bwd_prepare: per (token, head) row, delta*scale = scale*<dO, O> and lse*log2(e) into the
+//      workspace, and zero the fp32 dQ accumulator.
+//   2. ca_bwd_kernel: one workgroup of 8 waves per (task, block of 128 keys, kv head), in the
+//      order of the tile schedule.  K and V of the block sit in LDS for the workgroup's life.
+//      The query side (Q, dO and the two row statistics of every head of the kv group,
+//      flattened into rows like the forward) is streamed in blocks of 32 rows, starting at the
+//      first block the causal mask lets see these keys.  The waves form two groups of four;
+//      per iteration group 0 takes query block 2i and group 1 block 2i+1, so each SIMD always
+//      holds two waves at different points of the loop body and the MFMA pipe of one overlaps
+//      the VALU / LDS work of the other.  Within a group wave w owns keys 32w..32w+31:
+//        S = Q K^T, dP = dO V^T            A from the query tile, B from the K / V tiles (LDS)
+//        P = exp2(S*c - lse2), dS = P (dP*scale - delta*scale)          in registers
+//        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
+//                                          B = the accumulator registers converted to bf16
+//        dS -> LDS;  dQ[:, 32 columns of this wave] = dS K over the 128 keys -> fp32 atomics
+//      Query tiles are fetched two iterations ahead by LDS-direct global loads (no staging
+//      registers), one 256-byte row per instruction so the tile keeps its padded pitch.
+//      After the loop group 1 hands its dK^T / dV^T partial sums to group 0 through LDS.
 //   3. bwd_finish: dQ accumulator -> bf16 (and dK/dV when tasks alias KV rows).
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
@@ -29,10 +34,29 @@ namespace {
 
 constexpr int kPitch = 272;  // bytes per 128-element bf16 row in LDS
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kBwdThreads = 512;
+constexpr int kBN = kBwdKV;  // 128 keys per workgroup
+constexpr int kBM = kBwdRows;  // 32 flattened query rows per block
+
+// LDS map (bytes)
+constexpr int kKsOff = 0;
+constexpr int kVsOff = kKsOff + kBN * kPitch;
+constexpr int kTileOff = kVsOff + kBN * kPitch;
+constexpr int kTileQ = 0, kTileDO = kBM * kPitch;
+constexpr int kTileBytes = 2 * kBM * kPitch;                 // Q + dO of one block
+constexpr int kDsOff = kTileOff + 4 * kTileBytes;           // [stage 0/1][group 0/1]
+constexpr int kDsPitch = kBN * 2 + 16;
+constexpr int kDsBytes = kBM * kDsPitch;
+constexpr int kStatOff = kDsOff + 2 * kDsBytes;             // per (slot 0..2, group): lse2, dscaled, lim, rowoff
+constexpr int kStatBytes = 4 * kBM * 4;
+constexpr int kBwdLds = kStatOff + 6 * kStatBytes;
+constexpr int kRedBytes = 4 * 64 * 64 * 4;                  // group hand-over of one accumulator set
+static_assert(kRedBytes <= kTileOff, "reduction buffer must fit in the K/V region");
+static_assert(kBwdLds <= 160 * 1024, "LDS budget");
 
 struct BwdArgs {
   const __bf16 *q, *k, *v, *dout;
-  const float *lse, *delta;
+  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and delta*scale
   float *dq_acc;
   __bf16 *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
@@ -44,33 +68,30 @@ struct BwdArgs {
   float scale;
 };
 
-template <int KSUB, int MSUB>
-struct BwdLds {
-  static constexpr int kBN = kWaves * 32 * KSUB;
-  static constexpr int kBM = 32 * MSUB;
-  static constexpr int kDsPitch = kBN * 2 + 16;
-  static constexpr int kKs = 0;
-  static constexpr int kQs = kKs + kBN * kPitch;
-  static constexpr int kDOs = kQs + kBM * kPitch;
-  static constexpr int kDSs = kDOs + kBM * kPitch;
-  static constexpr int kLse = kDSs + kBM * kDsPitch;
-  static constexpr int kDelta = kLse + kBM * 4;
-  static constexpr int kLim = kDelta + kBM * 4;
-  static constexpr int kRowOff = kLim + kBM * 4;
-  static constexpr int kTotal = kRowOff + kBM * 4;
-};
+// One 16-byte piece per active lane from global memory straight into LDS at
+// lds_base + 16 * lane.  The compiler is not told this is a memory operation: the caller
+// orders it with wait_vm0() and a barrier before any wave reads the destination.  M0 is
+// written here and used by nothing else in these kernels.
+__device__ __forceinline__ uint32_t uniform32(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t voff, uint32_t lds_base) {
+  const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
+  const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbu), "s"(uniform32(lds_base)) : "memory");
+}
+__device__ __forceinline__ void lds_direct_load4(const void *gptr_lane, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
+}
+__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-template <int KSUB, int MSUB, bool ALIAS>
-__global__ __launch_bounds__(256, 1) void ca_bwd_kernel(BwdArgs a) {
-  using L = BwdLds<KSUB, MSUB>;
-  constexpr int kBN = L::kBN, kBM = L::kBM;
+template <bool ALIAS>
+__global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   const int item = blockIdx.x / a.hkv;
   if (item >= nitems) return;
   const int kvh = blockIdx.x - item * a.hkv;
-  const int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
-  const int task = it.x, nblk = it.y;
+  const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  const int task = it4.x, nblk = it4.y;
 
   const int q0 = a.cu_q[task];
   const int lq = a.cu_q[task + 1] - q0;
@@ -81,10 +102,12 @@ __global__ __launch_bounds__(256, 1) void ca_bwd_kernel(BwdArgs a) {
   const int nrows = lq * G;
   const int nmb = (nrows + kBM - 1) / kBM;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be so
+  const int grp = wave >> 2, kbw = wave & 3;
   const int l32 = lane & 31, g = lane >> 5;
-  const int kb0 = nblk * kBN;            // first key of the workgroup
-  const int kw0 = kb0 + wave * 32 * KSUB;  // first key of the wave
+  const int kb0 = nblk * kBN;      // first key of the workgroup
+  const int kw0 = kb0 + kbw * 32;  // first key of the wave
 
   int mb0 = 0;
   if (a.causal) {
@@ -92,278 +115,251 @@ __global__ __launch_bounds__(256, 1) void ca_bwd_kernel(BwdArgs a) {
     if (t_first < 0) t_first = 0;
     mb0 = (int)(((int64_t)t_first * G) / kBM);
   }
+  const int niter = nmb > mb0 ? (nmb - mb0 + 1) / 2 : 0;
 
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
-  const int64_t q_stride = (int64_t)a.hq * kHeadDim;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
 
-  // ---- K tile of the workgroup into LDS (row-major; read transposed for dQ)
+  // ---- K and V of the block into LDS (rows past the prefix as zeros)
   {
-    const int col = tid & 15, row = tid >> 4;
+    const int col = tid & 15, row = tid >> 4;  // 32 rows per pass
 #pragma unroll
-    for (int i = 0; i < kBN / 16; ++i) {
-      const int r = row + 16 * i;
+    for (int i = 0; i < kBN / 32; ++i) {
+      const int r = row + 32 * i;
       const int key = kb0 + r;
-      u32x4 val = u32x4{0, 0, 0, 0};
-      if (key < lk) val = *reinterpret_cast<const u32x4 *>(a.k + (int64_t)(ks + key) * kv_stride + kvh * kHeadDim + col * 8);
-      *reinterpret_cast<u32x4 *>(lds + L::kKs + r * kPitch + col * 16) = val;
-    }
-  }
-  // ---- K, V of this wave's keys as B operands (lane: key l32, d = 16s + 8g ..)
-  bf16x8 kfr[KSUB][8], vfr[KSUB][8];
-#pragma unroll
-  for (int kk = 0; kk < KSUB; ++kk) {
-    const int key = kw0 + kk * 32 + l32;
-    const bool ok = key < lk;
-    const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim + 8 * g;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      if (ok) {
-        kfr[kk][s] = *reinterpret_cast<const bf16x8 *>(a.k + off + 16 * s);
-        vfr[kk][s] = *reinterpret_cast<const bf16x8 *>(a.v + off + 16 * s);
-      } else {
-        kfr[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        vfr[kk][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      u32x4 kv = u32x4{0, 0, 0, 0}, vv = u32x4{0, 0, 0, 0};
+      if (key < lk) {
+        const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim + col * 8;
+        kv = *reinterpret_cast<const u32x4 *>(a.k + off);
+        vv = *reinterpret_cast<const u32x4 *>(a.v + off);
       }
+      *reinterpret_cast<u32x4 *>(lds + kKsOff + r * kPitch + col * 16) = kv;
+      *reinterpret_cast<u32x4 *>(lds + kVsOff + r * kPitch + col * 16) = vv;
     }
   }
 
-  f32x16 dkacc[KSUB][4], dvacc[KSUB][4];
+  f32x16 dkacc[4], dvacc[4];
 #pragma unroll
-  for (int kk = 0; kk < KSUB; ++kk)
+  for (int db = 0; db < 4; ++db)
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        dkacc[kk][db][r] = 0.f;
-        dvacc[kk][db][r] = 0.f;
-      }
-
-  // ---- query-side tile staging: kBM rows x 16 chunks of 16 B for Q and for dO
-  constexpr int kChunks = kBM * 16 / 256;  // per thread, per tensor
-  const int ld_col = tid & 15, ld_row = tid >> 4;
-  u32x4 qreg[kChunks], doreg[kChunks];
-  float lse_reg[kChunks], delta_reg[kChunks];
-  int lim_reg[kChunks], off_reg[kChunks];
-  const int64_t qbase = ((int64_t)q0 * a.hq + kvh * G) * kHeadDim;
-  auto load_tile = [&](int mb) {
-#pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-      const int r = mb * kBM + ld_row + 16 * i;
-      const int tok = r / G;
-      const int hg = r - tok * G;
-      const bool ok = r < nrows;
-      const int ro = tok * a.hq + hg;
-      if (ok) {
-        qreg[i] = *reinterpret_cast<const u32x4 *>(a.q + qbase + (int64_t)ro * kHeadDim + ld_col * 8);
-        doreg[i] = *reinterpret_cast<const u32x4 *>(a.dout + qbase + (int64_t)ro * kHeadDim + ld_col * 8);
-      } else {
-        qreg[i] = u32x4{0, 0, 0, 0};
-        doreg[i] = u32x4{0, 0, 0, 0};
-      }
-      if (ld_col == 0) {
-        int lm = a.causal ? tok + shift : lk - 1;
-        if (lm > lk - 1) lm = lk - 1;
-        if (ok) {
-          const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
-          lse_reg[i] = a.lse[so] * kLog2e;
-          delta_reg[i] = a.delta[so];
-          lim_reg[i] = lm;
-          off_reg[i] = ro;
-        } else {
-          lse_reg[i] = INFINITY;  // P = exp2(-inf) = 0 for rows past the task
-          delta_reg[i] = 0.f;
-          lim_reg[i] = 0x7fffffff;
-          off_reg[i] = -1;
-        }
-      }
+    for (int r = 0; r < 16; ++r) {
+      dkacc[db][r] = 0.f;
+      dvacc[db][r] = 0.f;
     }
-  };
-  auto store_tile = [&]() {
+
+  const int64_t qbase = ((int64_t)q0 * a.hq + kvh * G) * kHeadDim;  // element offset of (token q0, first head of the group)
+
+  // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block
+  auto issue_tile = [&](int stage, int slot, int mbx) {
+    const int tile = kTileOff + (stage * 2 + grp) * kTileBytes;
+    const int stat = kStatOff + (slot * 2 + grp) * kStatBytes;
+    // lanes 0..7 work out one row each; rows past the task are clamped to its last row so that
+    // the loads stay in bounds, and marked by lim = -1 / rowoff = -1
+    const int rl = kbw * 8 + (lane & 7);
+    const int rho = mbx * kBM + rl;
+    const bool ok = rho < nrows;
+    const int rc = ok ? rho : nrows - 1;
+    const int tok = rc / G;
+    const int hg = rc - tok * G;
+    const int ro = tok * a.hq + hg;
+    if (lane < 8) {
+      int lm = a.causal ? tok + shift : lk - 1;
+      if (lm > lk - 1) lm = lk - 1;
+      reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
+      reinterpret_cast<int *>(lds + stat + 3 * kBM * 4)[rl] = ok ? ro : -1;
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
+      lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
+      lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
+    }
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-      const int r = ld_row + 16 * i;
-      *reinterpret_cast<u32x4 *>(lds + L::kQs + r * kPitch + ld_col * 16) = qreg[i];
-      *reinterpret_cast<u32x4 *>(lds + L::kDOs + r * kPitch + ld_col * 16) = doreg[i];
-      if (ld_col == 0) {
-        reinterpret_cast<float *>(lds + L::kLse)[r] = lse_reg[i];
-        reinterpret_cast<float *>(lds + L::kDelta)[r] = delta_reg[i];
-        reinterpret_cast<int *>(lds + L::kLim)[r] = lim_reg[i];
-        reinterpret_cast<int *>(lds + L::kRowOff)[r] = off_reg[i];
+    for (int i = 0; i < 8; ++i) {
+      const int ro_i = __builtin_amdgcn_readlane(ro, i);
+      const __bf16 *qrow = a.q + qbase + (int64_t)ro_i * kHeadDim;
+      const __bf16 *dorow = a.dout + qbase + (int64_t)ro_i * kHeadDim;
+      const uint32_t dst = lds0 + tile + (kbw * 8 + i) * kPitch;
+      if (lane < 16) {
+        lds_direct_load16(qrow, lane * 16, dst + kTileQ);
+        lds_direct_load16(dorow, lane * 16, dst + kTileDO);
       }
     }
   };
 
   const float c = a.scale * kLog2e;
   // tile-independent LDS offsets
-  const int a_rd = l32 * kPitch + 16 * g;  // A operand rows (Q / dO / dS), + 32*s
+  const int a_rd = l32 * kPitch + 16 * g;                                                              // A operand rows, + 32*s
+  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;                                                 // B operand rows of K / V, + 32*s
   const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // transposed A
-  const int kt_rd = (8 * g + ((lane & 15) >> 2)) * kPitch + (16 * wave + 64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-  const int ds_rd = l32 * L::kDsPitch + 16 * g;
-  const int dq_col = 16 * wave + 64 * (l32 >> 4) + (l32 & 15);
+  const int kt_rd = (8 * g + ((lane & 15) >> 2)) * kPitch + (16 * kbw + 64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const int ds_rd = l32 * kDsPitch + 16 * g;
+  const int dq_col = 16 * kbw + 64 * (l32 >> 4) + (l32 & 15);
+  uint8_t *const dss = lds + kDsOff + grp * kDsBytes;
 
-  if (mb0 < nmb) {
-    load_tile(mb0);
-    store_tile();
-  }
-  __syncthreads();
+  // dQ of one iteration is added to global memory at the start of the next one: the
+  // vmcnt(0) wait that guards the tile then only ever waits for operations that are a whole
+  // iteration old.  The row statistics live in three slots so that the offsets an iteration
+  // needs for its deferred atomics survive the next tile fetch.
+  f32x16 dqacc;
+  float *const dqp = a.dq_acc + qbase + dq_col;
+  auto flush_dq = [&](int slot) {
+    const uint8_t *st = lds + kStatOff + (slot * 2 + grp) * kStatBytes;
+#pragma unroll
+    for (int cq = 0; cq < 4; ++cq) {
+      const i32x4 ro4 = *reinterpret_cast<const i32x4 *>(st + 3 * kBM * 4 + (8 * cq + 4 * g) * 4);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        if (ro4[rr] >= 0) unsafeAtomicAdd(dqp + (int64_t)ro4[rr] * kHeadDim, dqacc[4 * cq + rr]);
+    }
+  };
 
-  for (int mb = mb0; mb < nmb; ++mb) {
-    const bool has_next = mb + 1 < nmb;
-    if (has_next) load_tile(mb + 1);
+  if (niter > 0) issue_tile(0, 0, mb0 + grp);
+
+  int slot = 0;  // it % 3
+  for (int it = 0; it < niter; ++it) {
+    const int stage = it & 1;
+    wait_vm0();       // this wave's pieces of the current tile have landed
+    __syncthreads();  // ... and everybody else's; all readers of the other stage and of dS are done
+    if (it > 0) flush_dq(slot == 0 ? 2 : slot - 1);
+    if (it + 1 < niter) issue_tile(stage ^ 1, slot == 2 ? 0 : slot + 1, mb0 + 2 * (it + 1) + grp);
+
+    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+    const uint8_t *stat = lds + kStatOff + (slot * 2 + grp) * kStatBytes;
 
     // ---- S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys)
-    f32x16 sacc[MSUB][KSUB], dpacc[MSUB][KSUB];
+    f32x16 sacc, dpacc;
 #pragma unroll
-    for (int m = 0; m < MSUB; ++m)
-#pragma unroll
-      for (int kk = 0; kk < KSUB; ++kk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sacc[m][kk][r] = 0.f;
-          dpacc[m][kk][r] = 0.f;
-        }
+    for (int r = 0; r < 16; ++r) {
+      sacc[r] = 0.f;
+      dpacc[r] = 0.f;
+    }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-#pragma unroll
-      for (int m = 0; m < MSUB; ++m) {
-        const bf16x8 qa = *reinterpret_cast<const bf16x8 *>(lds + L::kQs + m * 32 * kPitch + a_rd + 32 * s);
-        const bf16x8 da = *reinterpret_cast<const bf16x8 *>(lds + L::kDOs + m * 32 * kPitch + a_rd + 32 * s);
-#pragma unroll
-        for (int kk = 0; kk < KSUB; ++kk) {
-          sacc[m][kk] = mfma32(qa, kfr[kk][s], sacc[m][kk]);
-          dpacc[m][kk] = mfma32(da, vfr[kk][s], dpacc[m][kk]);
-        }
-      }
+      const bf16x8 qa = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + a_rd + 32 * s);
+      const bf16x8 kb = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
+      const bf16x8 da = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + a_rd + 32 * s);
+      const bf16x8 vb = *reinterpret_cast<const bf16x8 *>(lds + kVsOff + b_rd + 32 * s);
+      sacc = mfma32(qa, kb, sacc);
+      dpacc = mfma32(da, vb, dpacc);
     }
 
     // ---- P and dS in registers; dS also to LDS for the dQ product
-    const int lim_first = reinterpret_cast<const int *>(lds + L::kLim)[0];
-    const bool need_mask = kw0 + 32 * KSUB - 1 > lim_first;
-    bf16x8 pb[MSUB][KSUB][2], dsb[MSUB][KSUB][2];
-#pragma unroll
-    for (int m = 0; m < MSUB; ++m) {
+    const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
+    const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
+    const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
+    bf16x8 pb[2], dsb[2];
+    {
 #pragma unroll
       for (int cq = 0; cq < 4; ++cq) {
-        const int qr = m * 32 + 8 * cq + 4 * g;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lds + L::kLse + qr * 4);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(lds + L::kDelta + qr * 4);
+        const int qr = 8 * cq + 4 * g;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
+        i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+        if (need_mask) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
 #pragma unroll
-        for (int kk = 0; kk < KSUB; ++kk) {
-#pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            const int r = 4 * cq + rr;
-            float p = fast_exp2(__builtin_fmaf(sacc[m][kk][r], c, -lse4[rr]));
-            if (need_mask) {
-              const int lm = reinterpret_cast<const int *>(lds + L::kLim)[qr + rr];
-              if (kw0 + kk * 32 + l32 > lm) p = 0.f;
-            }
-            const float ds = p * (dpacc[m][kk][r] - del4[rr]) * a.scale;
-            sacc[m][kk][r] = p;
-            dpacc[m][kk][r] = ds;
-          }
+        for (int rr = 0; rr < 4; ++rr) {
+          const int r = 4 * cq + rr;
+          float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
+          if (need_mask && kw0 + l32 > lim4[rr]) p = 0.f;
+          const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
+          sacc[r] = p;
+          dpacc[r] = ds;
         }
       }
-#pragma unroll
-      for (int kk = 0; kk < KSUB; ++kk) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int r0 = 8 * t;
-          pb[m][kk][t] = cvt8(sacc[m][kk][r0], sacc[m][kk][r0 + 1], sacc[m][kk][r0 + 2], sacc[m][kk][r0 + 3], sacc[m][kk][r0 + 4],
-                              sacc[m][kk][r0 + 5], sacc[m][kk][r0 + 6], sacc[m][kk][r0 + 7]);
-          dsb[m][kk][t] = cvt8(dpacc[m][kk][r0], dpacc[m][kk][r0 + 1], dpacc[m][kk][r0 + 2], dpacc[m][kk][r0 + 3],
-                               dpacc[m][kk][r0 + 4], dpacc[m][kk][r0 + 5], dpacc[m][kk][r0 + 6], dpacc[m][kk][r0 + 7]);
-        }
-        // dS[q][key] -> LDS, one bf16 per (lane, register)
-        __bf16 *dsp = reinterpret_cast<__bf16 *>(lds + L::kDSs) + (wave * 32 * KSUB + kk * 32 + l32);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dsp[(m * 32 + acc_row(r, g)) * (L::kDsPitch / 2)] = dsb[m][kk][r >> 3][r & 7];
-      }
-    }
-
-    // ---- dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the query rows)
-#pragma unroll
-    for (int m = 0; m < MSUB; ++m) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
+        const int r0 = 8 * t;
+        pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
+        dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
+      }
+      // dS[q][key] -> LDS, one bf16 per (lane, register)
+      __bf16 *dsp = reinterpret_cast<__bf16 *>(dss) + (kbw * 32 + l32);
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const int off = (m * 32 + 16 * t) * kPitch + t_rd + 32 * db;
-          const bf16x8 dot = cat4(lds_read_tr((const DISTCA_LDS void *)(lds + L::kDOs + off)),
-                                  lds_read_tr((const DISTCA_LDS void *)(lds + L::kDOs + off + 8 * kPitch)));
-          const bf16x8 qt = cat4(lds_read_tr((const DISTCA_LDS void *)(lds + L::kQs + off)),
-                                 lds_read_tr((const DISTCA_LDS void *)(lds + L::kQs + off + 8 * kPitch)));
+      for (int r = 0; r < 16; ++r) dsp[acc_row(r, g) * (kDsPitch / 2)] = dsb[r >> 3][r & 7];
+    }
+
+    // ---- dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows)
 #pragma unroll
-          for (int kk = 0; kk < KSUB; ++kk) {
-            dvacc[kk][db] = mfma32(dot, pb[m][kk][t], dvacc[kk][db]);
-            dkacc[kk][db] = mfma32(qt, dsb[m][kk][t], dkacc[kk][db]);
-          }
-        }
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const int off = 16 * t * kPitch + t_rd + 32 * db;
+        const bf16x8 dot = cat4(lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off)),
+                                lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off + 8 * kPitch)));
+        const bf16x8 qt = cat4(lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off)),
+                               lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off + 8 * kPitch)));
+        dvacc[db] = mfma32(dot, pb[t], dvacc[db]);
+        dkacc[db] = mfma32(qt, dsb[t], dkacc[db]);
       }
     }
-    __syncthreads();  // dS of every wave is in LDS; Q/dO tile no longer read
+    __syncthreads();  // dS of the four key waves is in LDS
 
-    // ---- dQ[:, this wave's 32 columns] = dS K over the workgroup's keys
+    // ---- dQ[:, this wave's 32 columns] = dS K over the workgroup's 128 keys
     {
-      f32x16 dqacc[MSUB];
 #pragma unroll
-      for (int m = 0; m < MSUB; ++m)
+      for (int r = 0; r < 16; ++r) dqacc[r] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dqacc[m][r] = 0.f;
-#pragma unroll 4
       for (int kstep = 0; kstep < kBN / 16; ++kstep) {
-        const uint8_t *kp = lds + L::kKs + kstep * 16 * kPitch + kt_rd;
+        const uint8_t *kp = lds + kKsOff + kstep * 16 * kPitch + kt_rd;
         const bf16x8 ktf = cat4(lds_read_tr((const DISTCA_LDS void *)kp), lds_read_tr((const DISTCA_LDS void *)(kp + 4 * kPitch)));
-#pragma unroll
-        for (int m = 0; m < MSUB; ++m) {
-          const bf16x8 dsa = *reinterpret_cast<const bf16x8 *>(lds + L::kDSs + m * 32 * L::kDsPitch + ds_rd + 32 * kstep);
-          dqacc[m] = mfma32(dsa, ktf, dqacc[m]);
-        }
+        const bf16x8 dsa = *reinterpret_cast<const bf16x8 *>(dss + ds_rd + 32 * kstep);
+        dqacc = mfma32(dsa, ktf, dqacc);
       }
-      float *dqp = a.dq_acc + qbase + dq_col;
-#pragma unroll
-      for (int m = 0; m < MSUB; ++m)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int ro = reinterpret_cast<const int *>(lds + L::kRowOff)[m * 32 + acc_row(r, g)];
-          if (ro >= 0) unsafeAtomicAdd(dqp + (int64_t)ro * kHeadDim, dqacc[m][r]);
-        }
     }
-    if (has_next) store_tile();
-    __syncthreads();
+    slot = slot == 2 ? 0 : slot + 1;
   }
+  if (niter > 0) flush_dq(slot == 0 ? 2 : slot - 1);
 
-  // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
+  // ---- group 1 hands its partial dK^T / dV^T to group 0 through LDS (K/V region, no longer read)
+  float *red = reinterpret_cast<float *>(lds) + (kbw * 64) * 64 + lane;
 #pragma unroll
-  for (int kk = 0; kk < KSUB; ++kk) {
-    const int key = kw0 + kk * 32 + l32;
-    if (key < lk) {
-      const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
+  for (int pass = 0; pass < 2; ++pass) {
+    __syncthreads();
+    if (grp == 1) {
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int cq = 0; cq < 4; ++cq) {
-          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          if (ALIAS) {
+        for (int r = 0; r < 16; ++r) red[(db * 16 + r) * 64] = pass == 0 ? dkacc[db][r] : dvacc[db][r];
+    }
+    __syncthreads();
+    if (grp == 0) {
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-              unsafeAtomicAdd(a.dk_acc + off + d0 + rr, dkacc[kk][db][4 * cq + rr]);
-              unsafeAtomicAdd(a.dv_acc + off + d0 + rr, dvacc[kk][db][4 * cq + rr]);
-            }
-          } else {
-            *reinterpret_cast<bf16x4 *>(a.dk + off + d0) =
-                cvt4(dkacc[kk][db][4 * cq], dkacc[kk][db][4 * cq + 1], dkacc[kk][db][4 * cq + 2], dkacc[kk][db][4 * cq + 3]);
-            *reinterpret_cast<bf16x4 *>(a.dv + off + d0) =
-                cvt4(dvacc[kk][db][4 * cq], dvacc[kk][db][4 * cq + 1], dvacc[kk][db][4 * cq + 2], dvacc[kk][db][4 * cq + 3]);
-          }
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (pass == 0) dkacc[db][r] += red[(db * 16 + r) * 64];
+          else dvacc[db][r] += red[(db * 16 + r) * 64];
         }
     }
   }
+
+  // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
+  const int key = kw0 + l32;
+  if (grp == 0 && key < lk) {
+    const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int cq = 0; cq < 4; ++cq) {
+        const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
+        if (ALIAS) {
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            unsafeAtomicAdd(a.dk_acc + off + d0 + rr, dkacc[db][4 * cq + rr]);
+            unsafeAtomicAdd(a.dv_acc + off + d0 + rr, dvacc[db][4 * cq + rr]);
+          }
+        } else {
+          *reinterpret_cast<bf16x4 *>(a.dk + off + d0) = cvt4(dkacc[db][4 * cq], dkacc[db][4 * cq + 1], dkacc[db][4 * cq + 2], dkacc[db][4 * cq + 3]);
+          *reinterpret_cast<bf16x4 *>(a.dv + off + d0) = cvt4(dvacc[db][4 * cq], dvacc[db][4 * cq + 1], dvacc[db][4 * cq + 2], dvacc[db][4 * cq + 3]);
+        }
+      }
+  }
 }
 
-// delta[h][t] = sum_d dO[t][h][d] * O[t][h][d]; also clears the fp32 dQ accumulator row.
+// Per (token, head) row: dscaled[h][t] = scale * sum_d dO*O and lse2[h][t] = lse[h][t]*log2(e);
+// also clears the row of the fp32 dQ accumulator.
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(const __bf16 *__restrict__ dout, const __bf16 *__restrict__ out,
-                                                         float *__restrict__ delta, float *__restrict__ dq_acc, int64_t rows,
-                                                         int32_t hq, int32_t total_q) {
+                                                         const float *__restrict__ lse, float *__restrict__ dscaled,
+                                                         float *__restrict__ lse2, float *__restrict__ dq_acc, int64_t rows,
+                                                         int32_t hq, int32_t total_q, float scale) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int sub = threadIdx.x & 15;
   float s = 0.f;
@@ -381,7 +377,9 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const __bf16 *__restri
   if (row < rows && sub == 0) {
     const int64_t t = row / hq;
     const int h = (int)(row - t * hq);
-    delta[(int64_t)h * total_q + t] = s;
+    const int64_t o = (int64_t)h * total_q + t;
+    dscaled[o] = s * scale;
+    lse2[o] = lse[o] * kLog2e;
   }
 }
 
@@ -403,13 +401,14 @@ __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float *__restrict__
 }
 
 struct BwdWorkspace {
-  int64_t sched, delta, dq_acc, dk_acc, dv_acc, total;
+  int64_t sched, delta, lse2, dq_acc, dk_acc, dv_acc, total;
 };
 BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias) {
   BwdWorkspace w;
   int64_t o = 0;
   w.sched = o; o += align_up(sched_bytes(p->num_tasks, bwd_max_items(p)), 256);
   w.delta = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
+  w.lse2 = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.dq_acc = o; o += align_up((int64_t)p->total_q * p->num_heads_q * kHeadDim * 4, 256);
   w.dk_acc = o; if (alias) o += align_up((int64_t)p->total_k * p->num_heads_kv * kHeadDim * 4, 256);
   w.dv_acc = o; if (alias) o += align_up((int64_t)p->total_k * p->num_heads_kv * kHeadDim * 4, 256);
@@ -480,11 +479,12 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
 
   const int64_t rows = (int64_t)p->total_q * p->num_heads_q;
   hipLaunchKernelGGL(bwd_prepare_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, (const __bf16 *)dout,
-                     (const __bf16 *)out, (float *)(ws + w.delta), (float *)(ws + w.dq_acc), rows, p->num_heads_q, p->total_q);
+                     (const __bf16 *)out, lse, (float *)(ws + w.delta), (float *)(ws + w.lse2), (float *)(ws + w.dq_acc), rows,
+                     p->num_heads_q, p->total_q, p->softmax_scale);
 
   BwdArgs a;
   a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v; a.dout = (const __bf16 *)dout;
-  a.lse = lse; a.delta = (const float *)(ws + w.delta); a.dq_acc = (float *)(ws + w.dq_acc);
+  a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta); a.dq_acc = (float *)(ws + w.dq_acc);
   a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
   a.dk_acc = alias ? (float *)(ws + w.dk_acc) : nullptr;
   a.dv_acc = alias ? (float *)(ws + w.dv_acc) : nullptr;
@@ -495,20 +495,19 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   const int64_t grid = max_items * p->num_heads_kv;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
-  using L = BwdLds<kBwdKsub, kBwdMsub>;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_kernel<kBwdKsub, kBwdMsub, false>, hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
-    hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_kernel<kBwdKsub, kBwdMsub, true>, hipFuncAttributeMaxDynamicSharedMemorySize, L::kTotal);
-    if (e1 != hipSuccess || e2 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS", L::kTotal);
+    hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    if (e1 != hipSuccess || e2 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS", kBwdLds);
     attr_set = true;
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     if (alias)
-      hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, true>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
+      hipLaunchKernelGGL((ca_bwd_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
     else
-      hipLaunchKernelGGL((ca_bwd_kernel<kBwdKsub, kBwdMsub, false>), dim3((unsigned)grid), dim3(256), L::kTotal, s, a);
+      hipLaunchKernelGGL((ca_bwd_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
   }
 
   hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(q_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dq_acc), (__bf16 *)dq, q_elems / 8);

@@ -19,18 +19,10 @@ constexpr int kFwdMsub = DISTCA_FWD_MSUB;
 constexpr int kFwdRows = kWaves * 32 * kFwdMsub;
 constexpr int kFwdKV = 64;
 
-// Backward: each wave owns BWD_KSUB sub-tiles of 32 keys; query rows are streamed in blocks
-// of 32 * BWD_MSUB flattened rows.
-#ifndef DISTCA_BWD_KSUB
-#define DISTCA_BWD_KSUB 1
-#endif
-#ifndef DISTCA_BWD_MSUB
-#define DISTCA_BWD_MSUB 1
-#endif
-constexpr int kBwdKsub = DISTCA_BWD_KSUB;
-constexpr int kBwdMsub = DISTCA_BWD_MSUB;
-constexpr int kBwdRows = 32 * kBwdMsub;
-constexpr int kBwdKV = kWaves * 32 * kBwdKsub;
+// Backward: a workgroup owns 128 keys (four waves of 32, in two copies that take alternate
+// query blocks); query rows are streamed in blocks of 32 flattened rows.
+constexpr int kBwdRows = 32;
+constexpr int kBwdKV = 128;
 
 inline int validate_params(const distca_ca_params *p) {
   if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: this build has kernels for head_dim 128 only", p->head_dim);
