@@ -24,6 +24,7 @@ HIPCC_FLAGS = [
     # (AGPR-form selection, the default above 256 registers, copies every accumulator the VALU
     # touches between the two files each loop iteration.)
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    "-munsafe-fp-atomics",  # float atomic add as one hardware instruction, not a CAS loop
     "-Wno-unused-command-line-argument",
 ]
 

@@ -68,7 +68,7 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-TIMER_CA_FWD, TIMER_CA_BWD, TIMER_MEMCPY_NON_CP, TIMER_MEMCPY_CP, TIMER_GRAD_SUM = range(5)
+TIMER_CA_FWD, TIMER_CA_BWD, TIMER_MEMCPY_NON_CP, TIMER_MEMCPY_CP, TIMER_GRAD_SUM, TIMER_CA_BWD_DQ = range(6)
 
 
 def timing_enable(on: bool) -> None:

@@ -3,26 +3,35 @@
 // Stands where the reference calls flash-attn's varlen backward
 // (distca/runtime/megatron/ops/fused_comm_attn.py:259-272).
 //
-// Launches on the caller's stream:
-//   1. bwd_prepare: per (token, head) row, delta*scale = scale*<dO, O> and lse*log2(e) into the
-//      workspace, and zero the fp32 dQ accumulator.
-//   2. ca_bwd_kernel: one workgroup of 8 waves per (task, block of 128 keys, kv head), in the
-//      order of the tile schedule.  K and V of the block sit in LDS for the workgroup's life.
-//      The query side (Q, dO and the two row statistics of every head of the kv group,
-//      flattened into rows like the forward) is streamed in blocks of 32 rows, starting at the
-//      first block the causal mask lets see these keys.  The waves form two groups of four;
-//      per iteration group 0 takes query block 2i and group 1 block 2i+1, so each SIMD always
-//      holds two waves at different points of the loop body and the MFMA pipe of one overlaps
-//      the VALU / LDS work of the other.  Within a group wave w owns keys 32w..32w+31:
+// The backward runs as two kernels that both recompute P from (Q, K, LSE), so that neither
+// needs floating-point atomics and the result is bit-reproducible (the `deterministic` switch
+// of the reference's FlashAttnArgs holds by construction).  A single-kernel form that added
+// dQ partial sums with fp32 atomics was measured first: the atomics alone (4 bytes per
+// (row, key) pair per 128 keys, 124 GB at 128K tokens) took as long as the rest of the kernel.
+//
+//   1. bwd_prepare_kernel: per (token, head) row, scale*<dO, O> and lse*log2(e) -> workspace.
+//   2. ca_bwd_dkdv_kernel: one workgroup of 8 waves per (task, block of 128 keys, kv head),
+//      in the order of the backward tile schedule.  K and V of the block sit in LDS for the
+//      workgroup's life.  The query side (Q, dO and the two row statistics of every head of
+//      the kv group, flattened into rows like the forward) is streamed in blocks of 32 rows
+//      from the first block the causal mask lets see these keys.  The waves form two groups of
+//      four; per iteration group 0 takes query block 2i and group 1 block 2i+1, so that every
+//      SIMD holds two waves at different points of the loop body.  In a group wave w owns
+//      keys 32w..32w+31:
 //        S = Q K^T, dP = dO V^T            A from the query tile, B from the K / V tiles (LDS)
 //        P = exp2(S*c - lse2), dS = P (dP*scale - delta*scale)          in registers
 //        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
 //                                          B = the accumulator registers converted to bf16
-//        dS -> LDS;  dQ[:, 32 columns of this wave] = dS K over the 128 keys -> fp32 atomics
-//      Query tiles are fetched two iterations ahead by LDS-direct global loads (no staging
-//      registers), one 256-byte row per instruction so the tile keeps its padded pitch.
-//      After the loop group 1 hands its dK^T / dV^T partial sums to group 0 through LDS.
-//   3. bwd_finish: dQ accumulator -> bf16 (and dK/dV when tasks alias KV rows).
+//      Query tiles arrive one iteration ahead through LDS-direct global loads, one 256-byte
+//      row per instruction so the tile keeps its padded pitch.  After the loop group 1 hands
+//      its partial sums to group 0 through LDS.
+//   3. ca_bwd_dq_kernel: one workgroup of 4 waves per (task, block of 128 flattened query
+//      rows, kv head), in the order of the forward tile schedule; the mirror image of the
+//      forward kernel.  Q and dO stay in registers as B operands, K/V tiles of 64 keys are
+//      streamed through LDS:
+//        S^T = K Q^T, dP^T = V dO^T        A from LDS rows, B from registers
+//        P, dS as above (one query row per lane: lse2 and delta are per-lane scalars)
+//        dQ^T += K^T dS^T                  A by transposing LDS reads of the K tile, B = dS registers
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 #include "api_util.h"
@@ -34,8 +43,12 @@ namespace {
 
 constexpr int kPitch = 272;  // bytes per 128-element bf16 row in LDS
 constexpr float kLog2e = 1.4426950408889634f;
+
+// ------------------------------------------------------------------------------------------
+// dK / dV
+// ------------------------------------------------------------------------------------------
 constexpr int kBwdThreads = 512;
-constexpr int kBN = kBwdKV;  // 128 keys per workgroup
+constexpr int kBN = kBwdKV;    // 128 keys per workgroup
 constexpr int kBM = kBwdRows;  // 32 flattened query rows per block
 
 // LDS map (bytes)
@@ -43,22 +56,18 @@ constexpr int kKsOff = 0;
 constexpr int kVsOff = kKsOff + kBN * kPitch;
 constexpr int kTileOff = kVsOff + kBN * kPitch;
 constexpr int kTileQ = 0, kTileDO = kBM * kPitch;
-constexpr int kTileBytes = 2 * kBM * kPitch;                 // Q + dO of one block
-constexpr int kDsOff = kTileOff + 4 * kTileBytes;           // [stage 0/1][group 0/1]
-constexpr int kDsPitch = kBN * 2 + 16;
-constexpr int kDsBytes = kBM * kDsPitch;
-constexpr int kStatOff = kDsOff + 2 * kDsBytes;             // per (slot 0..2, group): lse2, dscaled, lim, rowoff
-constexpr int kStatBytes = 4 * kBM * 4;
-constexpr int kBwdLds = kStatOff + 6 * kStatBytes;
-constexpr int kRedBytes = 4 * 64 * 64 * 4;                  // group hand-over of one accumulator set
+constexpr int kTileBytes = 2 * kBM * kPitch;      // Q + dO of one block
+constexpr int kStatOff = kTileOff + 4 * kTileBytes;  // tiles: [stage 0/1][group 0/1]
+constexpr int kStatBytes = 3 * kBM * 4;           // per (stage, group): lse2, dscaled, lim
+constexpr int kBwdLds = kStatOff + 4 * kStatBytes;
+constexpr int kRedBytes = 4 * 64 * 64 * 4;        // group hand-over of one accumulator set
 static_assert(kRedBytes <= kTileOff, "reduction buffer must fit in the K/V region");
 static_assert(kBwdLds <= 160 * 1024, "LDS budget");
 
 struct BwdArgs {
   const __bf16 *q, *k, *v, *dout;
   const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and delta*scale
-  float *dq_acc;
-  __bf16 *dk, *dv;
+  __bf16 *dq, *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;
@@ -68,23 +77,8 @@ struct BwdArgs {
   float scale;
 };
 
-// One 16-byte piece per active lane from global memory straight into LDS at
-// lds_base + 16 * lane.  The compiler is not told this is a memory operation: the caller
-// orders it with wait_vm0() and a barrier before any wave reads the destination.  M0 is
-// written here and used by nothing else in these kernels.
-__device__ __forceinline__ uint32_t uniform32(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
-__device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t voff, uint32_t lds_base) {
-  const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
-  const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbu), "s"(uniform32(lds_base)) : "memory");
-}
-__device__ __forceinline__ void lds_direct_load4(const void *gptr_lane, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
-}
-__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 template <bool ALIAS>
-__global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
+__global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   const int item = blockIdx.x / a.hkv;
@@ -150,11 +144,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
   const int64_t qbase = ((int64_t)q0 * a.hq + kvh * G) * kHeadDim;  // element offset of (token q0, first head of the group)
 
   // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block
-  auto issue_tile = [&](int stage, int slot, int mbx) {
+  auto issue_tile = [&](int stage, int mbx) {
     const int tile = kTileOff + (stage * 2 + grp) * kTileBytes;
-    const int stat = kStatOff + (slot * 2 + grp) * kStatBytes;
+    const int stat = kStatOff + (stage * 2 + grp) * kStatBytes;
     // lanes 0..7 work out one row each; rows past the task are clamped to its last row so that
-    // the loads stay in bounds, and marked by lim = -1 / rowoff = -1
+    // the loads stay in bounds, and marked by lim = -1 (every key masked)
     const int rl = kbw * 8 + (lane & 7);
     const int rho = mbx * kBM + rl;
     const bool ok = rho < nrows;
@@ -166,7 +160,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
       int lm = a.causal ? tok + shift : lk - 1;
       if (lm > lk - 1) lm = lk - 1;
       reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
-      reinterpret_cast<int *>(lds + stat + 3 * kBM * 4)[rl] = ok ? ro : -1;
       const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
       lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
       lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
@@ -186,43 +179,20 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
 
   const float c = a.scale * kLog2e;
   // tile-independent LDS offsets
-  const int a_rd = l32 * kPitch + 16 * g;                                                              // A operand rows, + 32*s
-  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;                                                 // B operand rows of K / V, + 32*s
+  const int a_rd = l32 * kPitch + 16 * g;                // A operand rows, + 32*s
+  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;   // B operand rows of K / V, + 32*s
   const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // transposed A
-  const int kt_rd = (8 * g + ((lane & 15) >> 2)) * kPitch + (16 * kbw + 64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-  const int ds_rd = l32 * kDsPitch + 16 * g;
-  const int dq_col = 16 * kbw + 64 * (l32 >> 4) + (l32 & 15);
-  uint8_t *const dss = lds + kDsOff + grp * kDsBytes;
 
-  // dQ of one iteration is added to global memory at the start of the next one: the
-  // vmcnt(0) wait that guards the tile then only ever waits for operations that are a whole
-  // iteration old.  The row statistics live in three slots so that the offsets an iteration
-  // needs for its deferred atomics survive the next tile fetch.
-  f32x16 dqacc;
-  float *const dqp = a.dq_acc + qbase + dq_col;
-  auto flush_dq = [&](int slot) {
-    const uint8_t *st = lds + kStatOff + (slot * 2 + grp) * kStatBytes;
-#pragma unroll
-    for (int cq = 0; cq < 4; ++cq) {
-      const i32x4 ro4 = *reinterpret_cast<const i32x4 *>(st + 3 * kBM * 4 + (8 * cq + 4 * g) * 4);
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr)
-        if (ro4[rr] >= 0) unsafeAtomicAdd(dqp + (int64_t)ro4[rr] * kHeadDim, dqacc[4 * cq + rr]);
-    }
-  };
+  if (niter > 0) issue_tile(0, mb0 + grp);
 
-  if (niter > 0) issue_tile(0, 0, mb0 + grp);
-
-  int slot = 0;  // it % 3
   for (int it = 0; it < niter; ++it) {
     const int stage = it & 1;
     wait_vm0();       // this wave's pieces of the current tile have landed
-    __syncthreads();  // ... and everybody else's; all readers of the other stage and of dS are done
-    if (it > 0) flush_dq(slot == 0 ? 2 : slot - 1);
-    if (it + 1 < niter) issue_tile(stage ^ 1, slot == 2 ? 0 : slot + 1, mb0 + 2 * (it + 1) + grp);
+    __syncthreads();  // ... and everybody else's; all readers of the other stage are done
+    if (it + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (it + 1) + grp);
 
     const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
-    const uint8_t *stat = lds + kStatOff + (slot * 2 + grp) * kStatBytes;
+    const uint8_t *stat = lds + kStatOff + (stage * 2 + grp) * kStatBytes;
 
     // ---- S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys)
     f32x16 sacc, dpacc;
@@ -241,39 +211,33 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
       dpacc = mfma32(da, vb, dpacc);
     }
 
-    // ---- P and dS in registers; dS also to LDS for the dQ product
+    // ---- P and dS in registers
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
     const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
     const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
     bf16x8 pb[2], dsb[2];
-    {
 #pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const int qr = 8 * cq + 4 * g;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
-        i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
-        if (need_mask) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
+    for (int cq = 0; cq < 4; ++cq) {
+      const int qr = 8 * cq + 4 * g;
+      const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
+      const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
+      i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+      if (need_mask) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int r = 4 * cq + rr;
-          float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
-          if (need_mask && kw0 + l32 > lim4[rr]) p = 0.f;
-          const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
-          sacc[r] = p;
-          dpacc[r] = ds;
-        }
+      for (int rr = 0; rr < 4; ++rr) {
+        const int r = 4 * cq + rr;
+        float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
+        if (need_mask && kw0 + l32 > lim4[rr]) p = 0.f;
+        const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
+        sacc[r] = p;
+        dpacc[r] = ds;
       }
+    }
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int r0 = 8 * t;
-        pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
-        dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
-      }
-      // dS[q][key] -> LDS, one bf16 per (lane, register)
-      __bf16 *dsp = reinterpret_cast<__bf16 *>(dss) + (kbw * 32 + l32);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dsp[acc_row(r, g) * (kDsPitch / 2)] = dsb[r >> 3][r & 7];
+    for (int t = 0; t < 2; ++t) {
+      const int r0 = 8 * t;
+      pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
+      dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
     }
 
     // ---- dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows)
@@ -290,23 +254,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
         dkacc[db] = mfma32(qt, dsb[t], dkacc[db]);
       }
     }
-    __syncthreads();  // dS of the four key waves is in LDS
-
-    // ---- dQ[:, this wave's 32 columns] = dS K over the workgroup's 128 keys
-    {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dqacc[r] = 0.f;
-#pragma unroll
-      for (int kstep = 0; kstep < kBN / 16; ++kstep) {
-        const uint8_t *kp = lds + kKsOff + kstep * 16 * kPitch + kt_rd;
-        const bf16x8 ktf = cat4(lds_read_tr((const DISTCA_LDS void *)kp), lds_read_tr((const DISTCA_LDS void *)(kp + 4 * kPitch)));
-        const bf16x8 dsa = *reinterpret_cast<const bf16x8 *>(dss + ds_rd + 32 * kstep);
-        dqacc = mfma32(dsa, ktf, dqacc);
-      }
-    }
-    slot = slot == 2 ? 0 : slot + 1;
   }
-  if (niter > 0) flush_dq(slot == 0 ? 2 : slot - 1);
 
   // ---- group 1 hands its partial dK^T / dV^T to group 0 through LDS (K/V region, no longer read)
   float *red = reinterpret_cast<float *>(lds) + (kbw * 64) * 64 + lane;
@@ -341,6 +289,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
       for (int cq = 0; cq < 4; ++cq) {
         const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
         if (ALIAS) {
+          // tasks that share KV rows add up here; the order of these additions is the one
+          // source of run-to-run variation, and only in the aliased-prefix form
 #pragma unroll
           for (int rr = 0; rr < 4; ++rr) {
             unsafeAtomicAdd(a.dk_acc + off + d0 + rr, dkacc[db][4 * cq + rr]);
@@ -354,12 +304,226 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_kernel(BwdArgs a) {
   }
 }
 
-// Per (token, head) row: dscaled[h][t] = scale * sum_d dO*O and lse2[h][t] = lse[h][t]*log2(e);
-// also clears the row of the fp32 dQ accumulator.
+// ------------------------------------------------------------------------------------------
+// dQ
+// ------------------------------------------------------------------------------------------
+constexpr int kDqKV = kFwdKV;  // 64 keys per tile
+constexpr int kDqStage = 2 * kDqKV * kPitch;  // K tile + V tile
+constexpr int kDqLds = 2 * kDqStage;
+
+template <int MSUB>
+__global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int nitems = a.sched[0];
+  const int item = blockIdx.x / a.hkv;
+  if (item >= nitems) return;
+  const int kvh = blockIdx.x - item * a.hkv;
+  const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  const int task = it4.x, mblk = it4.y;
+
+  const int q0 = a.cu_q[task];
+  const int lq = a.cu_q[task + 1] - q0;
+  const int lk = a.cu_k[task + 1] - a.cu_k[task];
+  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
+  const int G = a.group;
+  const int shift = lk - lq;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  constexpr int kRows = kWaves * 32 * MSUB;
+  const int row_wg = mblk * kRows;
+  const int nrows = lq * G;
+
+  int tok_end = (row_wg + kRows + G - 1) / G;
+  if (tok_end > lq) tok_end = lq;
+  int nvis = a.causal ? tok_end + shift : lk;
+  if (nvis > lk) nvis = lk;
+  const int ntiles = nvis > 0 ? (nvis + kDqKV - 1) / kDqKV : 0;
+
+  int row[MSUB], tok[MSUB], lim[MSUB];
+  bool valid[MSUB];
+  float lse2[MSUB], dsc[MSUB];
+  bf16x8 qf[MSUB][8], dof[MSUB][8];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+    row[m] = row_wg + (wave * MSUB + m) * 32 + l32;
+    valid[m] = row[m] < nrows;
+    tok[m] = row[m] / G;
+    const int hg = row[m] - tok[m] * G;
+    int lm = a.causal ? tok[m] + shift : lk - 1;
+    if (lm > lk - 1) lm = lk - 1;
+    lim[m] = lm;
+    const int64_t ro = ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim + 8 * g;
+    lse2[m] = INFINITY;  // rows past the task: P = exp2(-inf) = 0
+    dsc[m] = 0.f;
+    if (valid[m]) {
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
+      lse2[m] = a.lse2[so];
+      dsc[m] = a.dscaled[so];
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (valid[m]) {
+        qf[m][s] = *reinterpret_cast<const bf16x8 *>(a.q + ro + 16 * s);
+        dof[m][s] = *reinterpret_cast<const bf16x8 *>(a.dout + ro + 16 * s);
+      } else {
+        qf[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        dof[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  }
+  const int wrow0 = row_wg + wave * MSUB * 32;
+  int wrow1 = wrow0 + MSUB * 32 - 1;
+  if (wrow1 > nrows - 1) wrow1 = nrows - 1;
+  const bool wave_live = wrow0 < nrows;
+  int lim_first = 0x7fffffff, lim_last = -1;
+  if (wave_live) {
+    lim_first = a.causal ? wrow0 / G + shift : lk - 1;
+    if (lim_first > lk - 1) lim_first = lk - 1;
+    lim_last = a.causal ? wrow1 / G + shift : lk - 1;
+    if (lim_last > lk - 1) lim_last = lk - 1;
+  }
+
+  // ---- K/V tile staging: 64 rows x 16 chunks of 16 B, 4 chunks per thread and tensor
+  const int ld_col = tid & 15, ld_row = tid >> 4;
+  const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
+  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
+  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
+  u32x4 kreg[4], vreg[4];
+  auto load_tile = [&](int j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = j * kDqKV + ld_row + 16 * i;
+      if (key < lk) {
+        kreg[i] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)key * kv_stride);
+        vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + (int64_t)key * kv_stride);
+      } else {
+        kreg[i] = u32x4{0, 0, 0, 0};
+        vreg[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto store_tile = [&](int stage) {
+    uint8_t *kt = lds + stage * kDqStage;
+    uint8_t *vt = kt + kDqKV * kPitch;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = ld_row + 16 * i;
+      *reinterpret_cast<u32x4 *>(kt + r * kPitch + ld_col * 16) = kreg[i];
+      *reinterpret_cast<u32x4 *>(vt + r * kPitch + ld_col * 16) = vreg[i];
+    }
+  };
+
+  f32x16 dqacc[MSUB][4];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m)
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dqacc[m][db][r] = 0.f;
+  const float c = a.scale * kLog2e;
+  const int k_rd = l32 * kPitch + 16 * g;                                                                // + kb*32*kPitch + 32*s
+  const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // + (16t+8h)*kPitch + 32*db
+
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int stage = j & 1;
+    const uint8_t *kt = lds + stage * kDqStage;
+    const uint8_t *vt = kt + kDqKV * kPitch;
+    const bool has_next = j + 1 < ntiles;
+    if (has_next) load_tile(j + 1);
+
+    const int key0 = j * kDqKV;
+    const bool active = wave_live && key0 <= lim_last;
+    if (active) {
+      // ---- S^T = K Q^T, dP^T = V dO^T : [64 keys] x [32*MSUB rows]
+      f32x16 sacc[MSUB][2], dpacc[MSUB][2];
+#pragma unroll
+      for (int m = 0; m < MSUB; ++m)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            sacc[m][kb][r] = 0.f;
+            dpacc[m][kb][r] = 0.f;
+          }
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(kt + k_rd + kb * 32 * kPitch + 32 * s);
+          const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(vt + k_rd + kb * 32 * kPitch + 32 * s);
+#pragma unroll
+          for (int m = 0; m < MSUB; ++m) {
+            sacc[m][kb] = mfma32(kf, qf[m][s], sacc[m][kb]);
+            dpacc[m][kb] = mfma32(vf, dof[m][s], dpacc[m][kb]);
+          }
+        }
+      }
+      // ---- P, dS (one query row per lane) and the bf16 B operand of the dQ product
+      const bool need_mask = key0 + kDqKV - 1 > lim_first;
+      bf16x8 dsf[MSUB][4];
+#pragma unroll
+      for (int m = 0; m < MSUB; ++m) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, -lse2[m]));
+            if (need_mask && key0 + kb * 32 + acc_row(r, g) > lim[m]) p = 0.f;
+            dpacc[m][kb][r] = p * __builtin_fmaf(dpacc[m][kb][r], a.scale, -dsc[m]);
+          }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int kb = t >> 1, r0 = 8 * (t & 1);
+          dsf[m][t] = cvt8(dpacc[m][kb][r0], dpacc[m][kb][r0 + 1], dpacc[m][kb][r0 + 2], dpacc[m][kb][r0 + 3], dpacc[m][kb][r0 + 4],
+                           dpacc[m][kb][r0 + 5], dpacc[m][kb][r0 + 6], dpacc[m][kb][r0 + 7]);
+        }
+      }
+      // ---- dQ^T += K^T dS^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const uint8_t *kp = kt + t_rd + 16 * t * kPitch + 32 * db;
+          const bf16x8 ktf = cat4(lds_read_tr((const DISTCA_LDS void *)kp), lds_read_tr((const DISTCA_LDS void *)(kp + 8 * kPitch)));
+#pragma unroll
+          for (int m = 0; m < MSUB; ++m) dqacc[m][db] = mfma32(ktf, dsf[m][t], dqacc[m][db]);
+        }
+      }
+    }
+    if (has_next) store_tile(stage ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: dQ rows (bf16)
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+    if (valid[m]) {
+      const int hg = row[m] - tok[m] * G;
+      __bf16 *op = a.dq + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int cq = 0; cq < 4; ++cq) {
+          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
+          *reinterpret_cast<bf16x4 *>(op + d0) =
+              cvt4(dqacc[m][db][4 * cq], dqacc[m][db][4 * cq + 1], dqacc[m][db][4 * cq + 2], dqacc[m][db][4 * cq + 3]);
+        }
+    }
+  }
+}
+
+// Per (token, head) row: dscaled[h][t] = scale * sum_d dO*O and lse2[h][t] = lse[h][t]*log2(e).
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(const __bf16 *__restrict__ dout, const __bf16 *__restrict__ out,
                                                          const float *__restrict__ lse, float *__restrict__ dscaled,
-                                                         float *__restrict__ lse2, float *__restrict__ dq_acc, int64_t rows,
-                                                         int32_t hq, int32_t total_q, float scale) {
+                                                         float *__restrict__ lse2, int64_t rows, int32_t hq, int32_t total_q,
+                                                         float scale) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int sub = threadIdx.x & 15;
   float s = 0.f;
@@ -368,9 +532,6 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const __bf16 *__restri
     const bf16x8 b = *reinterpret_cast<const bf16x8 *>(out + row * kHeadDim + sub * 8);
 #pragma unroll
     for (int i = 0; i < 8; ++i) s += (float)a[i] * (float)b[i];
-    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-    *reinterpret_cast<f32x4 *>(dq_acc + row * kHeadDim + sub * 8) = z;
-    *reinterpret_cast<f32x4 *>(dq_acc + row * kHeadDim + sub * 8 + 4) = z;
   }
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
@@ -401,15 +562,15 @@ __global__ __launch_bounds__(256) void cvt_bf16_kernel(const float *__restrict__
 }
 
 struct BwdWorkspace {
-  int64_t sched, delta, lse2, dq_acc, dk_acc, dv_acc, total;
+  int64_t sched_kv, sched_q, delta, lse2, dk_acc, dv_acc, total;
 };
 BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias) {
   BwdWorkspace w;
   int64_t o = 0;
-  w.sched = o; o += align_up(sched_bytes(p->num_tasks, bwd_max_items(p)), 256);
+  w.sched_kv = o; o += align_up(sched_bytes(p->num_tasks, bwd_max_items(p)), 256);
+  w.sched_q = o; o += align_up(sched_bytes(p->num_tasks, fwd_max_items(p)), 256);
   w.delta = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.lse2 = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
-  w.dq_acc = o; o += align_up((int64_t)p->total_q * p->num_heads_q * kHeadDim * 4, 256);
   w.dk_acc = o; if (alias) o += align_up((int64_t)p->total_k * p->num_heads_kv * kHeadDim * 4, 256);
   w.dv_acc = o; if (alias) o += align_up((int64_t)p->total_k * p->num_heads_kv * kHeadDim * 4, 256);
   w.total = o;
@@ -442,15 +603,15 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
   int rc = validate_params(p);
   if (rc) return rc;
-  if (p->deterministic)
-    return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: deterministic=1 is not available (dQ is accumulated with float atomics)");
+  const bool alias = kv_off != nullptr;
+  if (p->deterministic && alias)
+    return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: deterministic=1 with kv_task_offsets (dK/dV of aliased rows are summed with float atomics)");
   if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv || !cu_q || !cu_k) {
-    if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
+    if (p->num_tasks == 0 || (p->total_q == 0 && p->total_k == 0)) return DISTCA_OK;
     return fail(DISTCA_E_INVALID, "ca_bwd: null pointer");
   }
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
     return fail(DISTCA_E_INVALID, "ca_bwd: tensors must be 16-byte aligned");
-  const bool alias = kv_off != nullptr;
   const BwdWorkspace w = bwd_layout(p, alias);
   if (!workspace || workspace_bytes < w.total)
     return fail(DISTCA_E_WORKSPACE, "ca_bwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)w.total);
@@ -460,7 +621,7 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   const int64_t kv_elems = (int64_t)p->total_k * p->num_heads_kv * kHeadDim;
   const int64_t q_elems = (int64_t)p->total_q * p->num_heads_q * kHeadDim;
 
-  // dk/dv rows no task reads must come back as zero
+  // rows no task touches must come back as zero
   if (kv_elems > 0) {
     if (alias) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 2)), dim3(256), 0, s, (u32x4 *)(ws + w.dk_acc),
@@ -472,48 +633,62 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   }
   if (p->num_tasks == 0 || p->total_q == 0) return check_launch("ca_bwd(clear)");
 
-  const SchedGeom geom = bwd_geom(p);
-  const int64_t max_items = bwd_max_items(p);
-  rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched), max_items, s);
-  if (rc) return rc;
-
   const int64_t rows = (int64_t)p->total_q * p->num_heads_q;
   hipLaunchKernelGGL(bwd_prepare_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, (const __bf16 *)dout,
-                     (const __bf16 *)out, lse, (float *)(ws + w.delta), (float *)(ws + w.lse2), (float *)(ws + w.dq_acc), rows,
-                     p->num_heads_q, p->total_q, p->softmax_scale);
+                     (const __bf16 *)out, lse, (float *)(ws + w.delta), (float *)(ws + w.lse2), rows, p->num_heads_q, p->total_q,
+                     p->softmax_scale);
 
   BwdArgs a;
   a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v; a.dout = (const __bf16 *)dout;
-  a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta); a.dq_acc = (float *)(ws + w.dq_acc);
-  a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
+  a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta);
+  a.dq = (__bf16 *)dq; a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
   a.dk_acc = alias ? (float *)(ws + w.dk_acc) : nullptr;
   a.dv_acc = alias ? (float *)(ws + w.dv_acc) : nullptr;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
-  a.sched = (const int32_t *)(ws + w.sched);
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
-  const int64_t grid = max_items * p->num_heads_kv;
-  if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
+
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    if (e1 != hipSuccess || e2 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS", kBwdLds);
+    hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipError_t e3 = hipFuncSetAttribute((const void *)ca_bwd_dq_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
+    if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve LDS");
     attr_set = true;
   }
+
+  // ---- dK, dV: one workgroup per (task, 128-key block, kv head)
   {
+    const SchedGeom geom = bwd_geom(p);
+    const int64_t max_items = bwd_max_items(p);
+    rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_kv), max_items, s);
+    if (rc) return rc;
+    const int64_t grid = max_items * p->num_heads_kv;
+    if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
+    a.sched = (const int32_t *)(ws + w.sched_kv);
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     if (alias)
-      hipLaunchKernelGGL((ca_bwd_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
+      hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
     else
-      hipLaunchKernelGGL((ca_bwd_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
+      hipLaunchKernelGGL((ca_bwd_dkdv_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
   }
-
-  hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(q_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dq_acc), (__bf16 *)dq, q_elems / 8);
+  // ---- dQ: one workgroup per (task, block of query rows, kv head)
+  {
+    const SchedGeom geom = fwd_geom(p);
+    const int64_t max_items = fwd_max_items(p);
+    rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
+    if (rc) return rc;
+    const int64_t grid = max_items * p->num_heads_kv;
+    if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
+    a.sched = (const int32_t *)(ws + w.sched_q);
+    ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
+    hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kDqLds, s, a);
+  }
   if (alias) {
     hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (__bf16 *)dk, kv_elems / 8);
     hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dv_acc), (__bf16 *)dv, kv_elems / 8);
   }
+  (void)q_elems;
   return check_launch("ca_bwd");
 }

@@ -11,9 +11,10 @@ namespace distca {
 constexpr int kHeadDim = 128;
 constexpr int kWaves = 4;  // waves per workgroup in every attention kernel
 
-// Forward: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles of 64 keys.
+// Forward and dQ kernels: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles
+// of 64 keys.  One sub-tile keeps a wave under 256 registers, so two workgroups share a CU.
 #ifndef DISTCA_FWD_MSUB
-#define DISTCA_FWD_MSUB 2
+#define DISTCA_FWD_MSUB 1
 #endif
 constexpr int kFwdMsub = DISTCA_FWD_MSUB;
 constexpr int kFwdRows = kWaves * 32 * kFwdMsub;

@@ -57,6 +57,22 @@ __device__ __forceinline__ bf16x4 cvt4(float a0, float a1, float a2, float a3) {
 __device__ __forceinline__ float pair_max(float x) { return __builtin_fmaxf(x, __shfl_xor(x, 32, 64)); }
 __device__ __forceinline__ float pair_sum(float x) { return x + __shfl_xor(x, 32, 64); }
 
+// LDS-direct global loads.  One piece per active lane goes from global memory straight into
+// LDS at lds_base + piece_bytes * lane, with no staging registers.  The compiler is not told
+// that these are memory operations: the caller orders them with wait_vm0() followed by a
+// barrier before any wave reads the destination.  M0 is written here and used by nothing
+// else in these kernels.
+__device__ __forceinline__ uint32_t uniform32(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t voff, uint32_t lds_base) {
+  const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
+  const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbu), "s"(uniform32(lds_base)) : "memory");
+}
+__device__ __forceinline__ void lds_direct_load4(const void *gptr_lane, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
+}
+__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -115,7 +115,8 @@ typedef struct distca_ca_params {
   int32_t max_seqlen_k; /* upper bound of any task's Lk                       */
   float softmax_scale;  /* multiplies q.k before softmax                      */
   int32_t causal;       /* 0 / 1                                              */
-  int32_t deterministic;/* backward only: 1 = no floating-point atomics       */
+  int32_t deterministic;/* backward only: 1 = refuse any path that uses float
+                           atomics (only the kv_task_offsets form does)       */
   int32_t reserved;
 } distca_ca_params;
 
@@ -168,11 +169,12 @@ int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
  * and clears them.  Not thread safe; leave disabled outside benchmarks.
  * ------------------------------------------------------------------------- */
 #define DISTCA_TIMER_CA_FWD 0      /* ca_fwd_kernel                          */
-#define DISTCA_TIMER_CA_BWD 1      /* ca_bwd_kernel                          */
+#define DISTCA_TIMER_CA_BWD 1      /* ca_bwd_dkdv_kernel                     */
 #define DISTCA_TIMER_MEMCPY_NON_CP 2
 #define DISTCA_TIMER_MEMCPY_CP 3
 #define DISTCA_TIMER_GRAD_SUM 4
-#define DISTCA_TIMER_COUNT 5
+#define DISTCA_TIMER_CA_BWD_DQ 5   /* ca_bwd_dq_kernel                       */
+#define DISTCA_TIMER_COUNT 6
 void distca_timing_enable(int on);
 int distca_timing_read(int which, double *total_ms, int64_t *launches);
 
