@@ -183,19 +183,10 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;   // B operand rows of K / V, + 32*s
   const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // transposed A
 
-  if (niter > 0) issue_tile(0, mb0 + grp);
-
-  for (int it = 0; it < niter; ++it) {
-    const int stage = it & 1;
-    wait_vm0();       // this wave's pieces of the current tile have landed
-    __syncthreads();  // ... and everybody else's; all readers of the other stage are done
-    if (it + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (it + 1) + grp);
-
+  f32x16 sacc, dpacc;
+  // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
+  auto phase_a = [&](int stage) {
     const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
-    const uint8_t *stat = lds + kStatOff + (stage * 2 + grp) * kStatBytes;
-
-    // ---- S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys)
-    f32x16 sacc, dpacc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       sacc[r] = 0.f;
@@ -210,8 +201,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       sacc = mfma32(qa, kb, sacc);
       dpacc = mfma32(da, vb, dpacc);
     }
-
-    // ---- P and dS in registers
+  };
+  // ---- phase B (VALU): P and dS in registers; phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
+  auto phase_bc = [&](int stage) {
+    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+    const uint8_t *stat = lds + kStatOff + (stage * 2 + grp) * kStatBytes;
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
     const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
     const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
@@ -239,8 +233,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
       dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
     }
-
-    // ---- dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 32 query rows)
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -254,6 +246,43 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
         dkacc[db] = mfma32(qt, dsb[t], dkacc[db]);
       }
     }
+  };
+
+  // The two groups run half a period apart: between the first and the second barrier of a
+  // period group 0 is in its MFMA-only phase A while group 1 starts with the VALU-heavy
+  // phase B; after the second barrier the roles swap.  A SIMD holds one wave of each
+  // group, so its MFMA pipe and its VALU are busy at the same time instead of by turns.
+  //   period p:  [barrier 1]  g0: A(p)          g1: B,C(p-1)
+  //              [barrier 2]  g0: B,C(p)        g1: A(p)
+  // A group's tile p+1 is requested right after the barrier that retires tile p-1 and is
+  // waited for before the same barrier one period later.
+  // Each group has its own copy of the loop (every wave still passes the same 2*(niter+1)
+  // barriers), which keeps the register allocation of either path as small as a single loop's.
+  if (niter > 0) issue_tile(0, mb0 + grp);
+  if (grp == 0) {
+    for (int p = 0; p < niter; ++p) {
+      const int stage = p & 1;
+      wait_vm0();
+      __syncthreads();
+      if (p + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (p + 1));
+      phase_a(stage);
+      __syncthreads();
+      phase_bc(stage);
+    }
+    __syncthreads();
+    __syncthreads();
+  } else {
+    __syncthreads();
+    for (int p = 0; p < niter; ++p) {
+      const int stage = p & 1;
+      wait_vm0();
+      __syncthreads();
+      if (p + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (p + 1) + 1);
+      phase_a(stage);
+      __syncthreads();
+      phase_bc(stage);
+    }
+    __syncthreads();
   }
 
   // ---- group 1 hands its partial dK^T / dV^T to group 0 through LDS (K/V region, no longer read)
