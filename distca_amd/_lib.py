@@ -11,7 +11,7 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("DISTCA_LIB_PATH") or os.path.join(_HERE, "libdistca_ca.so")
+LIB_PATH = os.path.join(_HERE, "libdistca_ca.so")
 
 ABI_VERSION = 1
 

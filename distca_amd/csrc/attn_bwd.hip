@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     // the loads stay in bounds, and marked by lim = -1 (every key masked)
     const int rl = kbw * 8 + (lane & 7);
     const int rho = mbx * kBM + rl;
-    const bool ok = rho < nrows;
+    const bool ok = rho < nrows && mbx >= mb0;  // a group's last block may not exist
     const int rc = ok ? rho : nrows - 1;
     const int tok = rc / G;
     const int hg = rc - tok * G;
@@ -192,14 +192,23 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       sacc[r] = 0.f;
       dpacc[r] = 0.f;
     }
+    // operands of step s+1 are requested before the MFMAs of step s are issued
+    bf16x8 qa[2], kb[2], da[2], vb[2];
+    auto load_a = [&](int s, int buf) {
+      qa[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + a_rd + 32 * s);
+      kb[buf] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
+      da[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + a_rd + 32 * s);
+      vb[buf] = *reinterpret_cast<const bf16x8 *>(lds + kVsOff + b_rd + 32 * s);
+    };
+    load_a(0, 0);
+    load_a(1, 1);
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const bf16x8 qa = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + a_rd + 32 * s);
-      const bf16x8 kb = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
-      const bf16x8 da = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + a_rd + 32 * s);
-      const bf16x8 vb = *reinterpret_cast<const bf16x8 *>(lds + kVsOff + b_rd + 32 * s);
-      sacc = mfma32(qa, kb, sacc);
-      dpacc = mfma32(da, vb, dpacc);
+      __builtin_amdgcn_sched_barrier(0);
+      sacc = mfma32(qa[s & 1], kb[s & 1], sacc);
+      dpacc = mfma32(da[s & 1], vb[s & 1], dpacc);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 2 < 8) load_a(s + 2, s & 1);
     }
   };
   // ---- phase B (VALU): P and dS in registers; phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
@@ -233,18 +242,23 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
       dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
     }
+    bf16x4 ct[2][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
+    auto load_c = [&](int j, int buf) {
+      const int off = 16 * (j >> 2) * kPitch + t_rd + 32 * (j & 3);
+      ct[buf][0] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off));
+      ct[buf][1] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off + 8 * kPitch));
+      ct[buf][2] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off));
+      ct[buf][3] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off + 8 * kPitch));
+    };
+    load_c(0, 0);
+    load_c(1, 1);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const int off = 16 * t * kPitch + t_rd + 32 * db;
-        const bf16x8 dot = cat4(lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off)),
-                                lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off + 8 * kPitch)));
-        const bf16x8 qt = cat4(lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off)),
-                               lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off + 8 * kPitch)));
-        dvacc[db] = mfma32(dot, pb[t], dvacc[db]);
-        dkacc[db] = mfma32(qt, dsb[t], dkacc[db]);
-      }
+    for (int j = 0; j < 8; ++j) {
+      __builtin_amdgcn_sched_barrier(0);
+      dvacc[j & 3] = mfma32(cat4(ct[j & 1][0], ct[j & 1][1]), pb[j >> 2], dvacc[j & 3]);
+      dkacc[j & 3] = mfma32(cat4(ct[j & 1][2], ct[j & 1][3]), dsb[j >> 2], dkacc[j & 3]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + 2 < 8) load_c(j + 2, j & 1);
     }
   };
 
@@ -258,13 +272,16 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // waited for before the same barrier one period later.
   // Each group has its own copy of the loop (every wave still passes the same 2*(niter+1)
   // barriers), which keeps the register allocation of either path as small as a single loop's.
-  if (niter > 0) issue_tile(0, mb0 + grp);
+  // Blocks are visited from the last one down to the diagonal: workgroups that run at the
+  // same time (neighbouring key blocks of one document, by the schedule) then read the same
+  // query rows at the same time and find them in their XCD's L2.
+  if (niter > 0) issue_tile(0, nmb - 1 - grp);
   if (grp == 0) {
     for (int p = 0; p < niter; ++p) {
       const int stage = p & 1;
       wait_vm0();
       __syncthreads();
-      if (p + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (p + 1));
+      if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 1 - 2 * (p + 1));
       phase_a(stage);
       __syncthreads();
       phase_bc(stage);
@@ -277,7 +294,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       const int stage = p & 1;
       wait_vm0();
       __syncthreads();
-      if (p + 1 < niter) issue_tile(stage ^ 1, mb0 + 2 * (p + 1) + 1);
+      if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 2 - 2 * (p + 1));
       phase_a(stage);
       __syncthreads();
       phase_bc(stage);
