@@ -48,8 +48,8 @@ def _compile(src: str, obj: str, extra: list[str]) -> None:
 
 
 def build_library(extra_flags: list[str] | None = None, verbose: bool = False, out_path: str | None = None) -> str:
-    """Compiles and links; `out_path` (default distca_amd/libdistca_ca.so) lets a tuning run
-    keep several variants side by side (select one with DISTCA_LIB_PATH)."""
+    """Compiles and links into `out_path` (default distca_amd/libdistca_ca.so, the only path
+    the loader reads)."""
     extra = list(extra_flags or [])
     lib_path = out_path or LIB_PATH
     obj_dir = os.path.join(PKG_DIR, "build", os.path.basename(lib_path))

@@ -1,0 +1,117 @@
+"""The C-ABI library loads without a GPU, exports every symbol include/distca_ca.h declares,
+and rejects bad arguments on the host before anything is launched."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from distca_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "distca_ca.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return sorted(set(re.findall(r"\b(distca_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "distca_ca.h"\nint main(void) { distca_ca_params p; (void)p; return 0; }\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src),
+                    "-o", str(tmp_path / "t.o")], check=True)
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = _declared_functions()
+    assert len(names) >= 12
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in distca_ca.h but not exported"
+    assert set(names) == set(_lib.SYMBOLS), "ctypes table and header disagree"
+
+
+def test_params_struct_layout_matches_header():
+    text = open(HEADER).read()
+    body = re.search(r"typedef struct distca_ca_params \{(.*?)\} distca_ca_params;", text, re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    body = re.sub(r"//[^\n]*", "", body)
+    fields = re.findall(r"(int32_t|float)\s+([a-z_]+)\s*;", body)
+    assert [f for _, f in fields] == [f for f, _ in _lib.CaParams._fields_]
+    assert ctypes.sizeof(_lib.CaParams) == 4 * len(fields)
+
+
+def test_abi_version_and_error_string():
+    lib = _lib.load()
+    assert lib.distca_abi_version() == _lib.ABI_VERSION
+    assert isinstance(lib.distca_last_error(), bytes)
+
+
+def _p(**kw):
+    base = dict(num_tasks=1, total_q=16, total_k=16, num_heads_q=32, num_heads_kv=8, head_dim=128,
+                max_seqlen_q=16, max_seqlen_k=16, softmax_scale=0.088, causal=1, deterministic=0, reserved=0)
+    base.update(kw)
+    return _lib.CaParams(*[base[f] for f, _ in _lib.CaParams._fields_])
+
+
+@pytest.mark.parametrize("bad", [dict(head_dim=64), dict(num_heads_q=30), dict(num_heads_kv=0), dict(num_tasks=-1),
+                                 dict(total_q=-5)])
+def test_unsupported_shapes_are_rejected_on_the_host(bad):
+    lib = _lib.load()
+    p = _p(**bad)
+    assert lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p)) < 0
+    # validation precedes any device call: with null pointers the call must return an error code
+    rc = lib.distca_ca_fwd(None, None, None, None, None, None, None, None, ctypes.byref(p), None, 0, None)
+    assert rc in (-1, -2)
+    assert lib.distca_last_error()
+
+
+def test_workspace_sizes_are_positive_and_monotone():
+    lib = _lib.load()
+    small = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(_p()))
+    big = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(_p(total_q=131072, total_k=131072, num_tasks=27,
+                                                              max_seqlen_q=65536, max_seqlen_k=65536)))
+    assert 0 < small < big
+    assert lib.distca_ca_fwd_workspace_bytes(ctypes.byref(_p())) > 0
+
+
+def test_pack_argument_checks_need_no_gpu():
+    lib = _lib.load()
+    # token size not a multiple of 16 bytes: rejected as the reference rejects it (memcpy.cu:246)
+    dummy = ctypes.create_string_buffer(64)        # host memory, never dereferenced: the size check comes first
+    a = ctypes.addressof(dummy)
+    assert lib.distca_memcpy_non_cp(a, a, a, a, None, 1, 24, 8, 1, None) < 0
+    assert b"16" in lib.distca_last_error()
+    assert lib.distca_memcpy_cp(a, a, a, a, a, 24, 8, 2, 1, 1, None) < 0
+    assert b"16" in lib.distca_last_error()
+    assert lib.distca_memcpy_non_cp(None, None, None, None, None, 1, 32, 8, 1, None) < 0
+    assert b"null" in lib.distca_last_error()
+    assert lib.distca_grad_sum(None, 99, None, None, None, 8, 128, 1, 1, None) < 0   # unknown dtype code
+    # zero-sized problems are no-ops that never touch the device
+    assert lib.distca_memcpy_non_cp(None, None, None, None, None, 0, 32, 0, 1, None) == 0
+
+
+def test_timing_api_without_launches():
+    lib = _lib.load()
+    ms, n = ctypes.c_double(-1), ctypes.c_int64(-1)
+    assert lib.distca_timing_read(99, ctypes.byref(ms), ctypes.byref(n)) < 0
+    lib.distca_timing_enable(0)
+    assert lib.distca_timing_read(0, ctypes.byref(ms), ctypes.byref(n)) == 0 and n.value == 0
+
+
+def test_schedule_host_reports_needed_capacity():
+    lib = _lib.load()
+    cu = np.array([0, 1000], dtype=np.int32)
+    p = _p(total_q=1000, total_k=1000, max_seqlen_q=1000, max_seqlen_k=1000)
+    n = lib.distca_ca_schedule_host(0, cu.ctypes.data, cu.ctypes.data, ctypes.byref(p), None, 0)
+    assert n > 0
+    small = np.full((2, 3), -7, dtype=np.int32)
+    # a short array receives the first max_items items; the full count is still returned
+    assert lib.distca_ca_schedule_host(0, cu.ctypes.data, cu.ctypes.data, ctypes.byref(p), small.ctypes.data, 1) == n
+    assert small[0, 0] == 0 and (small[1] == -7).all()

@@ -1,0 +1,124 @@
+"""Invariants of the tile scheduler, checked on the host mirror (distca_ca_schedule_host runs
+the same cost functions and the same bin sort as the device builder).
+
+The reference has no GPU-side scheduler to compare with; what is fixed is the mathematics:
+the items must tile every task exactly once, each item's extent must cover exactly the keys
+(or query blocks) the causal mask with KV-prefix offset lk - lq makes visible, and the order
+must be longest first."""
+import heapq
+
+import numpy as np
+import pytest
+
+from distca_amd import scheduler, workloads
+from oracle.attention import causal_pairs
+
+HQ, HKV = 32, 8
+G = HQ // HKV
+
+
+def _cu(lens):
+    return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+
+
+CASES = [
+    ([1], [1]),
+    ([5, 0, 300], [5, 7, 300]),
+    ([128, 64, 33], [128 + 512, 64, 33 + 1000]),          # KV prefixes (context-parallel shards)
+    ([31, 32, 33, 1000], [31, 32, 33, 1000]),
+    ([17, 600], [10, 600]),                               # lk < lq: the first tokens see nothing
+]
+
+
+@pytest.mark.parametrize("lq,lk", CASES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_items_tile_each_task_once_and_cover_visible_keys(lq, lk, causal):
+    rows, kv = scheduler.tile_shape(scheduler.FWD, HQ, HKV)
+    items = scheduler.build_schedule(scheduler.FWD, _cu(lq), _cu(lk), HQ, HKV, causal=causal)
+    seen = {}
+    for t, b, c in items.tolist():
+        assert (t, b) not in seen
+        seen[(t, b)] = c
+    for t, (a, k) in enumerate(zip(lq, lk)):
+        nblk = -(-a * G // rows)
+        assert sorted(b for (tt, b) in seen if tt == t) == list(range(nblk))
+        for b in range(nblk):
+            last_tok = min(a, -(-(b + 1) * rows // G)) - 1           # last token with a row in the block
+            vis = min(k, max(0, last_tok + 1 + (k - a))) if causal else k
+            assert seen[(t, b)] == -(-vis // kv)                       # KV tiles the block streams
+    costs = items[:, 2]
+    assert (np.diff(costs) <= 0).all()
+
+
+@pytest.mark.parametrize("lq,lk", CASES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_backward_items_cover_every_query_block_that_sees_the_key_block(lq, lk, causal):
+    rows, kv = scheduler.tile_shape(scheduler.BWD, HQ, HKV)
+    items = scheduler.build_schedule(scheduler.BWD, _cu(lq), _cu(lk), HQ, HKV, causal=causal)
+    seen = {(t, b): c for t, b, c in items.tolist()}
+    assert len(seen) == len(items)
+    for t, (a, k) in enumerate(zip(lq, lk)):
+        nkb = -(-k // kv) if a > 0 else 0
+        assert sorted(b for (tt, b) in seen if tt == t) == list(range(nkb))
+        nmb = -(-a * G // rows)
+        for n in range(nkb):
+            # brute force: query blocks holding a token that sees a key of block n
+            keys = np.arange(n * kv, min(k, (n + 1) * kv))
+            toks = np.arange(a)
+            vis_tok = toks[(toks + (k - a) >= keys.min())] if causal else toks
+            first = (int(vis_tok.min()) * G) // rows if len(vis_tok) else nmb
+            # the kernel walks m-blocks [nmb - cost, nmb): it must include `first`; it may start
+            # at most one block early (first-token rounding), never late
+            start = nmb - seen[(t, n)]
+            assert start <= first
+            assert first - start <= 1
+    assert (np.diff(items[:, 2]) <= 0).all()
+
+
+def test_forward_cost_totals_match_the_causal_pair_count():
+    """Sum of item costs x tile area bounds the exact pair count from above by at most the
+    diagonal tiles' slack (one KV tile and one row block per item)."""
+    b = workloads.config2_llama8b_128k()
+    rows, kv = scheduler.tile_shape(scheduler.FWD, HQ, HKV)
+    items = scheduler.build_schedule(scheduler.FWD, b.cu_seqlens_q, b.cu_seqlens_k, HQ, HKV)
+    lq, lk = np.diff(b.cu_seqlens_q), np.diff(b.cu_seqlens_k)
+    pairs = sum(causal_pairs(int(a), int(k)) for a, k in zip(lq, lk)) * G   # (row, key) pairs per kv head
+    covered = int(items[:, 2].astype(np.int64).sum()) * rows * kv
+    assert pairs <= covered <= pairs + len(items) * rows * kv + int(lq.sum()) * G * kv
+
+
+@pytest.mark.parametrize("kind", [scheduler.FWD, scheduler.BWD])
+def test_sorted_dispatch_balances_a_skewed_batch(kind):
+    """In-order dispatch of the sorted list onto free slots (what the hardware does with
+    workgroup ids) ends within a few percent of the mean load; unsorted order does not."""
+    b = workloads.config2_llama8b_128k()
+    items = scheduler.build_schedule(kind, b.cu_seqlens_q, b.cu_seqlens_k, HQ, HKV)
+    slots = 256 * 2 // HKV            # workgroup slots of the chip per kv head
+
+    def makespan(costs):
+        heap = [0] * slots
+        for c in costs:
+            heapq.heappush(heap, heapq.heappop(heap) + int(c) + 1)
+        return max(heap)
+
+    costs = items[:, 2]
+    ideal = (costs.sum() + len(costs)) / slots
+    assert makespan(costs) <= 1.05 * ideal + costs.max()
+    rng = np.random.default_rng(0)
+    assert makespan(costs) <= makespan(rng.permutation(costs))
+
+
+def test_empty_batch_and_empty_tasks():
+    assert scheduler.build_schedule(scheduler.FWD, [0], [0], HQ, HKV).shape == (0, 3)
+    items = scheduler.build_schedule(scheduler.FWD, _cu([0, 0, 4]), _cu([9, 0, 4]), HQ, HKV)
+    assert set(items[:, 0].tolist()) == {2}
+    items = scheduler.build_schedule(scheduler.BWD, _cu([0, 4]), _cu([700, 4]), HQ, HKV)
+    assert set(items[:, 0].tolist()) == {1}       # keys nobody queries receive no work item (their grads are the zero fill)
+
+
+def test_group_sizes():
+    for hq, hkv in [(8, 8), (16, 8), (64, 8), (28, 4)]:
+        rows, kv = scheduler.tile_shape(scheduler.FWD, hq, hkv)
+        items = scheduler.build_schedule(scheduler.FWD, _cu([100, 37]), _cu([100, 37]), hq, hkv)
+        g = hq // hkv
+        assert len(items) == -(-100 * g // rows) + -(-37 * g // rows)
