@@ -85,10 +85,20 @@ def _check_qkv(q: Tensor, k: Tensor, v: Tensor, cu_q: Tensor, cu_k: Tensor, kv_o
             raise RuntimeError("kv_task_offsets must be an int32 CUDA tensor of shape [num_tasks]")
 
 
+def _workspace(given: Optional[Tensor], need: int, device) -> Tensor:
+    if given is None:
+        return torch.empty((max(need, 16),), dtype=torch.uint8, device=device)
+    if given.dtype != torch.uint8 or not given.is_cuda or not given.is_contiguous() or given.numel() < need:
+        raise RuntimeError(f"workspace must be a contiguous uint8 CUDA tensor of at least {need} bytes")
+    return given
+
+
 def ca_varlen_fwd(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor, cu_seqlens_k: Tensor,
                   max_seqlen_q: int, max_seqlen_k: int, softmax_scale: Optional[float] = None, causal: bool = True,
-                  kv_task_offsets: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
-    """q [Tq,Hq,D], k,v [Tk,Hkv,D] bf16 -> (out [Tq,Hq,D] bf16, softmax_lse [Hq,Tq] fp32)."""
+                  kv_task_offsets: Optional[Tensor] = None, workspace: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """q [Tq,Hq,D], k,v [Tk,Hkv,D] bf16 -> (out [Tq,Hq,D] bf16, softmax_lse [Hq,Tq] fp32).
+    `workspace` (uint8 CUDA tensor of at least distca_ca_fwd_workspace_bytes) is allocated
+    per call when omitted."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
     tq, hq, d = q.shape
     tk, hkv, _ = k.shape
@@ -100,7 +110,7 @@ def ca_varlen_fwd(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor, cu_seql
         _lib.check(int(need), "ca_varlen_fwd")
     out = torch.empty_like(q)
     lse = torch.empty((hq, tq), dtype=torch.float32, device=q.device)
-    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    ws = _workspace(workspace, int(need), q.device)
     with torch.cuda.device(q.device):
         rc = lib.distca_ca_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
                                cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
@@ -114,7 +124,8 @@ def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, so
                   cu_seqlens_q: Tensor, cu_seqlens_k: Tensor, max_seqlen_q: int, max_seqlen_k: int,
                   softmax_scale: Optional[float] = None, causal: bool = True, deterministic: bool = False,
                   kv_task_offsets: Optional[Tensor] = None,
-                  dq: Optional[Tensor] = None, dk: Optional[Tensor] = None, dv: Optional[Tensor] = None):
+                  dq: Optional[Tensor] = None, dk: Optional[Tensor] = None, dv: Optional[Tensor] = None,
+                  workspace: Optional[Tensor] = None):
     """Gradients (dq, dk, dv) in bf16; written into dq/dk/dv when given (the reference's
     flash-attn backward fills caller-allocated tensors, fused_comm_attn.py:236,259-272)."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
@@ -140,7 +151,7 @@ def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, so
     for name, t, ref in (("dq", dq, q), ("dk", dk, k), ("dv", dv, v)):
         if t.shape != ref.shape or t.dtype != torch.bfloat16 or not t.is_contiguous() or not t.is_cuda:
             raise RuntimeError(f"{name} must be a contiguous bfloat16 CUDA tensor shaped like its input")
-    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    ws = _workspace(workspace, int(need), q.device)
     with torch.cuda.device(q.device):
         rc = lib.distca_ca_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),

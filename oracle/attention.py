@@ -159,10 +159,13 @@ def ca_reference_rows(
     cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequence[int], task: int, row0: int, row1: int,
     softmax_scale: Optional[float] = None, causal: bool = True,
     kv_task_offsets: Optional[Sequence[int]] = None, dtype: torch.dtype = torch.float32,
+    out_rows: Optional[torch.Tensor] = None, lse_rows: Optional[torch.Tensor] = None,
 ):
     """Rows [row0,row1) of one task against its full KV prefix: (out, lse, dq) for those
     rows (dq None without dout).  Used to spot-check long tasks whose full fp32
-    evaluation would take hours on host cores; same formulas as above."""
+    evaluation would take hours on host cores; same formulas as above.  With `out_rows`
+    [rows, Hq, D] and `lse_rows` [Hq, rows] the gradient is formed from those saved forward
+    results, as ca_reference_bwd does with out= / softmax_lse=."""
     hq, d = q.shape[1], q.shape[2]
     g = hq // k.shape[1]
     scale = softmax_scale if softmax_scale is not None else d ** -0.5
@@ -178,8 +181,10 @@ def ca_reference_rows(
     dqb = None
     if dout is not None:
         dob = dout[q0 + row0:q0 + row1].to(dtype).permute(1, 0, 2)
-        delta = (dob * ob).sum(-1, keepdim=True)
-        ds = p * (torch.matmul(dob, vb.transpose(1, 2)) - delta)
+        o_used = ob if out_rows is None else out_rows.to(dtype).permute(1, 0, 2)
+        p_used = p if lse_rows is None else torch.nan_to_num(torch.exp(s - lse_rows.to(dtype).unsqueeze(-1)), nan=0.0)
+        delta = (dob * o_used).sum(-1, keepdim=True)
+        ds = p_used * (torch.matmul(dob, vb.transpose(1, 2)) - delta)
         dqb = (torch.matmul(ds, kb) * scale).permute(1, 0, 2)
     return ob.permute(1, 0, 2), l.squeeze(-1), dqb
 

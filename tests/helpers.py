@@ -53,3 +53,25 @@ def assert_close_bf16(got, ref, what, max_abs=MAX_ABS_TOL, mean_rel=MEAN_REL_TOL
 
 def cu(lens):
     return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+
+
+def task_sums(a, b, cu, hkv):
+    """(sum of a*b, sum of (a*b)^2) per (task, kv head) in fp64; query heads fold onto their kv head."""
+    t, h, d = a.shape
+    prod = a.double() * b.double()
+    per_tok = torch.stack([prod.sum(2), (prod * prod).sum(2)], 0).reshape(2, t, hkv, h // hkv).sum(3)   # [2, T, hkv]
+    csum = torch.cat([torch.zeros_like(per_tok[:, :1]), per_tok.cumsum(1)], 1)
+    idx = torch.as_tensor(np.asarray(cu), device=a.device, dtype=torch.long)
+    seg = csum[:, idx[1:]] - csum[:, idx[:-1]]
+    return seg[0].cpu(), seg[1].cpu()
+
+
+def assert_identity(lhs, rhs, what):
+    """Both sides are sums of products of bf16-rounded kernel outputs with exact inputs: every
+    product carries an independent relative error of up to 2^-8 (output rounding, plus the bf16
+    rounding of P and dS ahead of the MFMAs), so the sums agree to a few standard deviations of
+    2^-8 * sqrt(sum of squared products).  8 sigma allowed."""
+    (a, a2), (b, b2) = lhs, rhs
+    tol = 8 * 2.0 ** -8 * torch.sqrt(a2 + b2) + 1e-6
+    bad = (a - b).abs() > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} (task, kv head) cells off, worst {((a - b).abs() / tol).max().item():.1f} x tol"

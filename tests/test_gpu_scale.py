@@ -1,0 +1,200 @@
+"""Full-size runs of the benchmark workloads, checked through properties that do not need the
+full fp32 oracle (which would take hours on host cores at these sizes):
+
+  * sampled query rows against the oracle (out, lse, dq for those rows over the whole prefix);
+  * <V, dV> = <O, dO>  (O is linear in V) and  <Q, dQ> = <K, dK>  (scores depend on Q K^T only,
+    so scaling Q or K by 1+eps moves the loss equally), per kv head;
+  * two runs give bit-identical results (no atomics anywhere in the unaliased path);
+  * a document served as prefix tasks equals the same document served whole;
+  * the schedule the device built is the one the host mirror predicts.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close_bf16, assert_identity, randn_bf16, task_sums
+from oracle.attention import ca_reference_rows
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev_inputs(batch, hq, hkv, cuda, seed):
+    """Seeded N(0,1) bf16 inputs generated on the device (host generation of 10^9 values is slow)."""
+    d = 128
+    tq, tk = batch.total_q, batch.kv_rows
+    g = torch.Generator(device=cuda).manual_seed(seed)
+    rnd = lambda *shape: torch.randn(shape, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v, do = rnd(tq, hq, d), rnd(tk, hkv, d), rnd(tk, hkv, d), rnd(tq, hq, d)
+    cu_q = torch.tensor(batch.cu_seqlens_q, dtype=torch.int32, device=cuda)
+    cu_k = torch.tensor(batch.cu_seqlens_k, dtype=torch.int32, device=cuda)
+    return q, k, v, do, cu_q, cu_k
+
+
+def _fwd_bwd(batch, hq, hkv, cuda, seed=0):
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    q, k, v, do, cu_q, cu_k = _dev_inputs(batch, hq, hkv, cuda, seed)
+    mq, mk = int(max(batch.q_lens)), int(max(batch.k_lens))
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk)
+    dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk)
+    torch.cuda.synchronize()
+    return q, k, v, do, out, lse, dq, dk, dv
+
+
+def _rows_ref(batch, q, k, v, do, t, r0, r1, out=None, lse=None):
+    """Oracle (out, lse, dq) of rows [r0, r1) of task t; only that task's slices leave the device."""
+    q0, q1 = int(batch.cu_seqlens_q[t]), int(batch.cu_seqlens_q[t + 1])
+    k0, k1 = int(batch.cu_seqlens_k[t]), int(batch.cu_seqlens_k[t + 1])
+    k1 -= (q1 - q0) - r1            # keys beyond the last sampled row's horizon are masked anyway
+    q1 = q0 + r1
+    return ca_reference_rows(q[q0:q1].cpu(), k[k0:k1].cpu(), v[k0:k1].cpu(), None if do is None else do[q0:q1].cpu(),
+                             [0, q1 - q0], [0, k1 - k0], 0, r0, r1,
+                             out_rows=None if out is None else out[q0 + r0:q0 + r1].cpu(),
+                             lse_rows=None if lse is None else lse[:, q0 + r0:q0 + r1].cpu())
+
+
+def _check_sampled_rows(batch, q, k, v, do, out, lse, dq, rng, n_samples=6, rows=16):
+    lens = np.asarray(batch.q_lens)
+    tasks = list(np.argsort(lens)[-2:]) + list(rng.choice(len(lens), size=n_samples - 2))
+    for t in tasks:
+        lq = int(lens[t])
+        if lq == 0:
+            continue
+        r0 = int(rng.integers(0, max(1, lq - rows + 1)))
+        r1 = min(lq, r0 + rows)
+        if t == tasks[0]:
+            r0, r1 = lq - min(rows, lq), lq                   # the longest rows of the longest task
+        # the gradient oracle consumes the (out, lse) the backward kernel was handed
+        o_ref, l_ref, dq_ref = _rows_ref(batch, q, k, v, do, int(t), r0, r1, out, lse)
+        g0 = int(batch.cu_seqlens_q[t]) + r0
+        sl = slice(g0, g0 + (r1 - r0))
+        print(f"  rows task={t} [{r0},{r1}) of {lq}", flush=True)
+        assert_close_bf16(out[sl], o_ref, f"out task {t}")
+        assert (lse[:, sl].cpu() - l_ref).abs().max().item() <= 2e-3
+        assert_close_bf16(dq[sl], dq_ref, f"dq task {t}")
+
+
+def test_config2_llama8b_128k_properties(cuda):
+    """The benchmark workload at full size: 131072 packed tokens, 32q/8kv heads."""
+    from distca_amd import workloads
+    b = workloads.config2_llama8b_128k()
+    print("cfg2 fwd+bwd", flush=True)
+    q, k, v, do, out, lse, dq, dk, dv = _fwd_bwd(b, 32, 8, cuda)
+    for name, t in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert torch.isfinite(t.float()).all(), name
+    _check_sampled_rows(b, q, k, v, do, out, lse, dq, np.random.default_rng(0))
+    # linearity identities per (task, kv head)
+    cu = b.cu_seqlens_q
+    assert_identity(task_sums(v, dv, cu, 8), task_sums(out, do, cu, 8), "<V,dV> = <O,dO>")
+    assert_identity(task_sums(q, dq, cu, 8), task_sums(k, dk, cu, 8), "<Q,dQ> = <K,dK>")
+    print("cfg2 second run (bit reproducibility)", flush=True)
+    again = _fwd_bwd(b, 32, 8, cuda)
+    for name, x, y in zip(("out", "lse", "dq", "dk", "dv"), (out, lse, dq, dk, dv), again[4:]):
+        assert torch.equal(x, y), f"{name} differs between two identical runs"
+
+
+def test_config5_llama70b_heads_forward_rows(cuda):
+    """64q/8kv heads (group 8) with one 262144-token document among short ones: forward at
+    full size, rows of the long document and of short ones against the oracle."""
+    from distca_amd import workloads
+    from distca_amd.fused_comm_attn import ca_varlen_fwd
+    b = workloads.config5_llama70b_skewed()
+    q, k, v, do, cu_q, cu_k = _dev_inputs(b, 64, 8, cuda, 40)
+    print("cfg5 fwd", flush=True)
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, int(max(b.q_lens)), int(max(b.k_lens)))
+    torch.cuda.synchronize()
+    big = int(np.argmax(b.q_lens))
+    for t, r0 in ((big, int(b.q_lens[big]) - 8), (big, 100000), (0 if big else 1, 0)):
+        r1 = min(int(b.q_lens[t]), r0 + 8)
+        print(f"  rows task={t} [{r0},{r1})", flush=True)
+        o_ref, l_ref, _ = _rows_ref(b, q, k, v, None, t, r0, r1)
+        g0 = int(b.cu_seqlens_q[t]) + r0
+        assert_close_bf16(out[g0:g0 + r1 - r0], o_ref, f"out task {t}")
+        assert (lse[:, g0:g0 + r1 - r0].cpu() - l_ref).abs().max().item() <= 2e-3
+
+
+def test_prefix_tasks_equal_whole_document(cuda):
+    """One 24576-token document as 6 CA tasks over a shared KV copy == the document served whole,
+    forward and backward (dK/dV of the shared rows are summed across tasks on device)."""
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    n, hq, hkv = 24576, 32, 8
+    cuts = [0, 2048, 6144, 7000, 13000, 20480, n]
+    q = randn_bf16((n, hq, 128), 1).to(cuda); k = randn_bf16((n, hkv, 128), 2).to(cuda)
+    v = randn_bf16((n, hkv, 128), 3).to(cuda); do = randn_bf16((n, hq, 128), 4).to(cuda)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=cuda)
+    whole = i32([0, n])
+    print("whole document", flush=True)
+    out_w, lse_w = ca_varlen_fwd(q, k, v, whole, whole, n, n)
+    dq_w, dk_w, dv_w = ca_varlen_bwd(do, q, k, v, out_w, lse_w, whole, whole, n, n)
+    cu_q = i32(cuts)
+    cu_k = i32([0] + list(np.cumsum(cuts[1:])))           # task i sees keys [0, cuts[i+1])
+    kv_off = i32([0] * (len(cuts) - 1))
+    print("prefix tasks", flush=True)
+    mq, mk = int(np.diff(cuts).max()), n
+    out_s, lse_s = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+    dq_s, dk_s, dv_s = ca_varlen_bwd(do, q, k, v, out_s, lse_s, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+    torch.cuda.synchronize()
+    assert_close_bf16(out_s, out_w.float(), "out")
+    assert (lse_s - lse_w).abs().max().item() <= 2e-3
+    assert_close_bf16(dq_s, dq_w.float(), "dq", max_abs=3e-2)
+    assert_close_bf16(dk_s, dk_w.float(), "dk", max_abs=3e-2)
+    assert_close_bf16(dv_s, dv_w.float(), "dv", max_abs=3e-2)
+
+
+@pytest.mark.parametrize("kind", ["fwd", "bwd"])
+def test_device_schedule_equals_host_mirror(cuda, kind):
+    """The workspace begins with the schedule the device built ([0] = item count, then the
+    per-task block prefix, then (task, block, cost, 0) items): same items, same order of cost
+    bins as distca_ca_schedule_host."""
+    from distca_amd import scheduler, workloads
+    from distca_amd._lib import CaParams, load
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    import ctypes
+    rng = np.random.default_rng(4)
+    ql = rng.integers(1, 3000, size=14).astype(np.int64); ql[3] = 0
+    b = workloads.TaskBatch("prefix_tasks", ql, ql + rng.integers(0, 4000, size=14) * (rng.random(14) < 0.6), 32, 8)
+    hq, hkv = 32, 8
+    q, k, v, do, cu_q, cu_k = _dev_inputs(b, hq, hkv, cuda, 9)
+    mq, mk = int(max(b.q_lens)), int(max(b.k_lens))
+    p = CaParams(len(b.q_lens), b.total_q, b.kv_rows, hq, hkv, 128, mq, mk, 128 ** -0.5, 1, 0, 0)
+    lib = load()
+    nbytes = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+    ws = torch.zeros((nbytes,), dtype=torch.uint8, device=cuda)
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, workspace=ws)
+    if kind == "bwd":
+        ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, workspace=ws)
+    torch.cuda.synchronize()
+    w = ws.cpu().view(torch.int32).numpy()
+    host = scheduler.build_schedule(scheduler.BWD if kind == "bwd" else scheduler.FWD, b.cu_seqlens_q, b.cu_seqlens_k, hq, hkv)
+    n = int(w[0])
+    assert n == len(host)
+    header = (4 + len(b.q_lens) + 1 + 3) // 4 * 4
+    items = w[header:header + 4 * n].reshape(n, 4)
+    assert (items[:, 3] == 0).all()
+    dev = items[:, :3]
+    assert (np.diff(dev[:, 2]) <= 0).all()
+    as_set = lambda a: sorted(map(tuple, a.tolist()))
+    assert as_set(dev) == as_set(host)
+    assert np.array_equal(dev[:, 2], host[:, 2])          # identical cost sequence; ties may permute
+
+
+def test_pack_round_trip_full_size(cuda):
+    """cfg4 at full size: pack then unpack returns the source bit for bit, q-sized and k-sized tokens."""
+    from distca_amd import workloads
+    from distca_amd.ops import a2a_memcpy_non_cp
+    lay = workloads.config4_pack()
+    for hidden in (4096, 1024):
+        tb = hidden * 2
+        lens = torch.tensor(lay.seq_tokens, dtype=torch.int64)
+        sizes = lens * tb
+        perm = torch.randperm(len(lens), generator=torch.Generator().manual_seed(3))
+        off = torch.zeros(len(lens), dtype=torch.int64)
+        off[perm] = torch.cumsum(sizes[perm], 0) - sizes[perm]
+        src = torch.randint(-32768, 32767, (lay.num_tokens, hidden), dtype=torch.int16, device=cuda).view(torch.bfloat16)
+        buf = torch.zeros(int(sizes.sum()), dtype=torch.uint8, device=cuda)
+        a2a_memcpy_non_cp(src, off.to(cuda), lens.to(cuda), True, buffer=buf)
+        back = torch.zeros_like(src)
+        a2a_memcpy_non_cp(back, off.to(cuda), lens.to(cuda), False, buffer=buf)
+        torch.cuda.synchronize()
+        assert torch.equal(back.view(torch.int16), src.view(torch.int16))
+        # a checksum of the buffer equals the checksum of the source: every byte landed exactly once
+        assert int(buf.view(torch.int16).to(torch.int64).sum()) == int(src.view(torch.int16).to(torch.int64).sum())

@@ -1,0 +1,179 @@
+"""One tick of the CA server on explicit buffers (fused_comm_attn.py:298-461 of the
+reference): unpack shards -> attention -> pack the reply, forward and backward, checked
+byte for byte against the pack oracle and numerically against whole-document attention.
+
+Layout under test: a 600-token document cut into query shards a|b|c (200, 150, 250 tokens)
+served as three CA tasks with KV prefixes a, a+b, a+b+c, plus a whole 130-token document.
+The receive buffer holds each K/V shard once; the unpack offsets of a prefix's shards alias
+them (as the reference's metadata does), so the server materialises one KV copy per task,
+and the backward sums the copies' gradients into the main copy before the masked pack."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close_bf16, make_qkv
+from oracle import fa2a
+from oracle.attention import ca_reference_bwd, ca_reference_fwd
+
+pytestmark = pytest.mark.gpu
+
+HQ, HKV, D = 6, 2, 128            # lse row = 24 bytes: exercises the pad of [out | lse] to 16 bytes
+QB, KB = HQ * D * 2, HKV * D * 2
+SH = [200, 150, 250]              # shards of document 0
+DOC1 = 130
+
+
+def _layout():
+    q_lens = SH + [DOC1]
+    # K shards in task order: task a: [a]; b: [a, b]; c: [a, b, c]; doc1: [d]
+    k_shard_src = [0, 0, 1, 0, 1, 2, 3]                    # which stored shard each one reads
+    stored = SH + [DOC1]
+    k_lens_shard = [stored[s] for s in k_shard_src]
+    k_lens_task = [200, 350, 600, DOC1]
+    return q_lens, k_shard_src, stored, k_lens_shard, k_lens_task
+
+
+def _offsets(sizes, rng, gap=16):
+    """Scattered, non-overlapping, 16-byte aligned regions in a random order."""
+    off = np.zeros(len(sizes), np.int64)
+    cur = 0
+    for i in rng.permutation(len(sizes)):
+        off[i] = cur
+        cur += sizes[i] + gap * int(rng.integers(0, 4))
+    return off, cur
+
+
+def _dev(x, cuda, dtype=None):
+    t = torch.as_tensor(np.asarray(x))
+    return (t.to(dtype) if dtype else t).to(cuda)
+
+
+def test_server_tick_forward_and_backward(cuda):
+    from distca_amd.fused_comm_attn import (FlashAttnArgs, PackedSeqParams, ServerBwdMeta, ServerFwdMeta,
+                                            ca_server_backward, ca_server_forward)
+    from distca_amd.utils import size_pad_by_int4
+    rng = np.random.default_rng(11)
+    q_lens, k_src, stored, k_lens_shard, k_lens_task = _layout()
+    tq, tk_stored = sum(q_lens), sum(stored)
+    q, k, v, do = make_qkv(tq, tk_stored, HQ, HKV, D, 21)          # bf16 CPU, [T, H, D]
+    q2, k2, v2 = (x.reshape(x.shape[0], -1) for x in (q, k, v))
+    stored_start = np.concatenate([[0], np.cumsum(stored)])
+
+    # ---- receive buffer as the all-to-all would leave it: q shards, stored k, stored v ----
+    sizes = [n * QB for n in q_lens] + [n * KB for n in stored] * 2
+    off, nbytes = _offsets(sizes, rng)
+    q_off, ks_off, vs_off = off[:4], off[4:8], off[8:12]
+    recv = np.full(nbytes, 0xAB, np.uint8)
+    fa2a.copy_non_cp(q2.view(torch.uint8).numpy(), recv, q_off, q_lens)
+    fa2a.copy_non_cp(k2.view(torch.uint8).numpy(), recv, ks_off, stored)
+    fa2a.copy_non_cp(v2.view(torch.uint8).numpy(), recv, vs_off, stored)
+    k_off = np.array([ks_off[s] for s in k_src]); v_off = np.array([vs_off[s] for s in k_src])
+
+    out_tb, _ = size_pad_by_int4(HQ * D * 2 + HQ * 4, 1)
+    assert out_tb == 1568
+    so, send_bytes = _offsets([n * out_tb for n in q_lens], rng)
+    send = torch.full((send_bytes,), 0xCD, dtype=torch.uint8, device=cuda)
+    cu_q = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(k_lens_task)]).astype(np.int32)
+    fa_params = PackedSeqParams(_dev(cu_q, cuda), _dev(cu_k, cuda), max(q_lens), max(k_lens_task))
+    fa_args = FlashAttnArgs(HQ, HKV, D)
+    meta = ServerFwdMeta(_dev(q_lens, cuda, torch.int64), _dev(k_lens_shard, cuda, torch.int64),
+                         _dev(q_off, cuda), _dev(k_off, cuda), _dev(v_off, cuda),
+                         _dev(q_lens, cuda, torch.int64), _dev(so, cuda),
+                         (tq, HQ * D), (sum(k_lens_shard), HKV * D))
+    print("server forward", flush=True)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, meta, fa_params, fa_args)
+    torch.cuda.synchronize()
+
+    # numerics: three prefix tasks == whole-document causal attention
+    cu_doc = np.array([0, 600, 730], np.int32)
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_doc, cu_doc)
+    assert_close_bf16(out.reshape(tq, HQ, D), ref_out, "out")
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
+
+    # bytes: the send buffer is exactly the pack of [out | lse^T | pad] and nothing else moved
+    tok = np.zeros((tq, out_tb), np.uint8)
+    tok[:, :HQ * D * 2] = out.cpu().view(torch.uint8).numpy()
+    tok[:, HQ * D * 2:HQ * D * 2 + HQ * 4] = lse.T.contiguous().cpu().view(torch.uint8).numpy().reshape(tq, -1)
+    expect = np.full(send_bytes, 0xCD, np.uint8)
+    fa2a.copy_non_cp(tok, expect, so, q_lens)
+    assert np.array_equal(send.cpu().numpy(), expect)
+
+    # ---- backward request: merged [dO | O | lse | q | pad] tokens + the same K/V shards ----
+    mt, _ = size_pad_by_int4(3 * HQ * D * 2 + HQ * 4, 1)
+    merged = np.zeros((tq, mt), np.uint8)
+    parts = [do.reshape(tq, -1).view(torch.uint8).numpy(), out.cpu().view(torch.uint8).numpy(),
+             lse.T.contiguous().cpu().view(torch.uint8).numpy().reshape(tq, -1), q2.view(torch.uint8).numpy()]
+    c = 0
+    for p_ in parts:
+        merged[:, c:c + p_.shape[1]] = p_; c += p_.shape[1]
+    sizes = [n * mt for n in q_lens] + [n * KB for n in stored] * 2
+    off, nbytes = _offsets(sizes, rng)
+    mq_off, ks_off, vs_off = off[:4], off[4:8], off[8:12]
+    recv = np.full(nbytes, 0x11, np.uint8)
+    fa2a.copy_non_cp(merged, recv, mq_off, q_lens)
+    fa2a.copy_non_cp(k2.view(torch.uint8).numpy(), recv, ks_off, stored)
+    fa2a.copy_non_cp(v2.view(torch.uint8).numpy(), recv, vs_off, stored)
+    k_off = np.array([ks_off[s] for s in k_src]); v_off = np.array([vs_off[s] for s in k_src])
+
+    # gradient reply: dq shards, then one dk and one dv region per stored shard (main copies only)
+    shard_start = np.concatenate([[0], np.cumsum(k_lens_shard)])
+    main_of = {}
+    main_mask = np.zeros(len(k_src), np.int8)
+    for i, s in enumerate(k_src):
+        if s not in main_of:
+            main_of[s] = i; main_mask[i] = 1
+    copies = {i: [j for j, s in enumerate(k_src) if main_of[s] == i and j != i] for i in main_of.values()}
+    max_copies = max(len(c_) for c_ in copies.values())
+    num_copies = np.zeros(len(k_src), np.int32)
+    copy_start = np.zeros((len(k_src), max_copies), np.int64)
+    for i, js in copies.items():
+        num_copies[i] = len(js)
+        copy_start[i, :len(js)] = [shard_start[j] for j in js]
+    sizes = [n * QB for n in q_lens] + [n * KB for n in stored] * 2
+    goff, gbytes = _offsets(sizes, rng)
+    dq_off = goff[:4]
+    dk_off = np.array([goff[4 + s] for s in k_src]); dv_off = np.array([goff[8 + s] for s in k_src])
+    gsend = torch.full((gbytes,), 0x77, dtype=torch.uint8, device=cuda)
+    bmeta = ServerBwdMeta(_dev(q_lens, cuda, torch.int64), _dev(k_lens_shard, cuda, torch.int64),
+                          _dev(mq_off, cuda), _dev(k_off, cuda), _dev(v_off, cuda),
+                          _dev(q_lens, cuda, torch.int64), _dev(k_lens_shard, cuda, torch.int64),
+                          _dev(dq_off, cuda), _dev(dk_off, cuda), _dev(dv_off, cuda),
+                          _dev(main_mask, cuda), _dev(num_copies, cuda), _dev(copy_start, cuda),
+                          (tq, HQ * D), (tq, HQ), (sum(k_lens_shard), HKV * D))
+    print("server backward", flush=True)
+    dq, dk, dv = ca_server_backward(torch.from_numpy(recv).to(cuda), gsend, bmeta, fa_args, fa_params.cu_seqlens_q,
+                                    fa_params.cu_seqlens_kv, max(q_lens), max(k_lens_task))
+    torch.cuda.synchronize()
+
+    # numerics against the whole-document gradient: dq directly, dk/dv = the main copies after the sum
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=out.cpu().reshape(tq, HQ, D),
+                                              softmax_lse=lse.cpu())
+    assert_close_bf16(dq.reshape(tq, HQ, D), ref_dq, "dq")
+    main_rows = np.concatenate([np.arange(shard_start[main_of[s]], shard_start[main_of[s]] + stored[s]) for s in range(4)])
+    # up to three bf16 roundings on the way (each task's output, then one per summed copy) where a
+    # single kernel has one: tolerances 4e-2 / 3e-3 here instead of 2e-2 / 1e-3
+    assert_close_bf16(dk[main_rows].reshape(-1, HKV, D), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
+    assert_close_bf16(dv[main_rows].reshape(-1, HKV, D), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
+
+    # bytes: reply buffer == masked pack of what the server returned; unmasked copies sent nothing
+    expect = np.full(gbytes, 0x77, np.uint8)
+    fa2a.copy_non_cp(dq.cpu().view(torch.uint8).numpy(), expect, dq_off, q_lens)
+    fa2a.copy_non_cp(dk.cpu().view(torch.uint8).numpy(), expect, dk_off, k_lens_shard, main_mask)
+    fa2a.copy_non_cp(dv.cpu().view(torch.uint8).numpy(), expect, dv_off, k_lens_shard, main_mask)
+    assert np.array_equal(gsend.cpu().numpy(), expect)
+
+
+def test_grad_sum_matches_oracle_on_attention_gradients(cuda):
+    """The duplicate-gradient sum on device is bit-exact with the oracle's per-copy rounding."""
+    from distca_amd.ops import pre_a2a_grad_acc
+    g = torch.Generator().manual_seed(5)
+    lens = [200, 200, 150, 200, 150, 250]
+    data = (torch.randn((sum(lens), HKV * D), generator=g) * 3).to(torch.bfloat16)
+    num_copies = [2, 0, 1, 0, 0, 0]
+    starts = [[200, 550], [0, 0], [750, 0], [0, 0], [0, 0], [0, 0]]
+    want = data.clone()
+    fa2a.grad_sum(want, num_copies, starts, lens)
+    got = data.to(cuda)
+    pre_a2a_grad_acc(got, _dev(num_copies, cuda, torch.int32), _dev(starts, cuda, torch.int64), _dev(lens, cuda, torch.int64))
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))

@@ -8,7 +8,9 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from helpers import cu
+import pytest
+
+from helpers import cu, make_qkv
 from oracle.attention import (attention_flops, ca_reference_bwd, ca_reference_fwd, ca_reference_rows, causal_pairs)
 
 
@@ -201,3 +203,23 @@ def test_pair_count_and_flops():
     assert causal_pairs(3, 7) == 3 * 7 - 3  # rows see 5, 6, 7 keys
     fwd, bwd = attention_flops(cu([512, 1024, 2560]), cu([512, 1024, 2560]), 32, 128)
     assert fwd == 4 * 32 * 128 * 3934208 and bwd == 10 * 32 * 128 * 3934208
+
+
+def test_linearity_identities_hold_and_catch_a_dropped_tile():
+    """<V,dV> = <O,dO> and <Q,dQ> = <K,dK> per (task, kv head) for bf16-rounded oracle results;
+    removing one 64-key tile's contribution to dV of a 300-token task breaks the first."""
+    from helpers import assert_identity, task_sums
+    q_lens = [300, 70]
+    q, k, v, do = make_qkv(370, 370, 4, 2, 128, 3)
+    out, lse = ca_reference_fwd(q, k, v, cu(q_lens), cu(q_lens))
+    dq, dk, dv = ca_reference_bwd(do, q, k, v, cu(q_lens), cu(q_lens))
+    r = lambda x: x.to(torch.bfloat16)
+    c = cu(q_lens)
+    assert_identity(task_sums(v, r(dv), c, 2), task_sums(r(out), do, c, 2), "vdv")
+    assert_identity(task_sums(q, r(dq), c, 2), task_sums(k, r(dk), c, 2), "qdq")
+    # dV without the contribution of query rows 128..255 to keys 64..127 (one tile of one head group)
+    _, _, dv_part = ca_reference_bwd(do[128:256], q[128:256], k[:256], v[:256], [0, 128], [0, 256])
+    broken = dv.clone()
+    broken[64:128] -= dv_part[64:128]
+    with pytest.raises(AssertionError):
+        assert_identity(task_sums(v, r(broken), c, 2), task_sums(r(out), do, c, 2), "vdv")
