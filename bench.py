@@ -9,9 +9,13 @@ before the timed region.  One JSON line is printed on stdout; a human-readable t
 to stderr.
 
 Algorithmic work: causal pairs P = sum_tasks [Lq*Lk - Lq(Lq-1)/2]; forward 4*Hq*D*P FLOP,
-backward 10*Hq*D*P FLOP.  `roofline` describes the dominant kernel (the attention backward
-kernel) with its launch duration measured live by HIP events the library records on the
-launch stream.  `cpu_baseline` times the CPU oracle (per-document fp32 PyTorch attention,
+backward 10*Hq*D*P FLOP.  `roofline` describes the dominant kernels, the two that make up the
+attention backward (ca_bwd_dkdv_kernel over key blocks, ca_bwd_dq_kernel over query blocks):
+algorithmic backward FLOPs over the sum of their launch durations, measured live by HIP events
+the library records on the launch stream.  Both recompute S and dP, so together they execute
+14*Hq*D*P FLOP for 10*Hq*D*P of algorithmic work; `executed_tflops` reports that rate per kernel.
+`traffic` is the HBM bytes per backward (both kernels) measured once with rocprofv3 --pmc on
+the default workload and scaled by a copy kernel of known size; null for other sizes.  `cpu_baseline` times the CPU oracle (per-document fp32 PyTorch attention,
 forward + backward) on this box's host cores over a bounded sample of the same documents.
 """
 from __future__ import annotations
@@ -29,6 +33,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
+# WRITE_SIZE (x1.000), factors from the pack kernel's known copy size in the same run
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 22.17e9, "ca_bwd_dkdv_kernel": 47.01e9, "ca_bwd_dq_kernel": 20.47e9}
 
 
 def log(*a):
@@ -126,6 +133,7 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     batch = config2_llama8b_128k(total=args.tokens)
+    default_workload = args.tokens == 131072
     hq, hkv, d = batch.num_heads_q, batch.num_heads_kv, batch.head_dim
     tq = batch.total_q
     flop_fwd, flop_bwd = batch.flops()
@@ -196,8 +204,11 @@ def main():
                    "causal_pairs": batch.causal_pairs, "flop_fwd": flop_fwd, "flop_bwd": flop_bwd,
                    "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2)},
         "roofline": {"bound": "mfma", "kernel": "ca_bwd_dkdv_kernel + ca_bwd_dq_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(bwd_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(bwd_tf / PEAK_BF16_TFLOPS, 4),
+                     "traffic": (MEASURED_TRAFFIC_BYTES["ca_bwd_dkdv_kernel"] + MEASURED_TRAFFIC_BYTES["ca_bwd_dq_kernel"]) if default_workload else None,
+                     "traffic_unit": "bytes per launch (both kernels)",
                      "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv_kernel": round(dkdv_k, 4), "ca_bwd_dq_kernel": round(dq_k, 4)},
+                     "executed_tflops": {"ca_bwd_dkdv_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
                      "launches": bwd_n,
                      "also": {"ca_fwd_kernel": {"achieved": round(fwd_tf, 2), "frac": round(fwd_tf / PEAK_BF16_TFLOPS, 4),
                                                 "avg_launch_ms": round(fwd_k, 4), "launches": fwd_n}}},
