@@ -1,0 +1,234 @@
+"""Types that carry lengths, offsets and masks into the CA-server path, and a single-rank
+plan builder.
+
+`SeqLens`, `LogicalShape` and `DedupGradSumMetadata` have the fields and the dtype
+normalisation of distca/runtime/metadata.py:12-67 (lengths and offsets int64, masks int8,
+num_copies int32, cu_seqlens int32 as in runtime/megatron/packed_seq_params.py:11-14).
+`get_attn_metadata` follows runtime/compute_metadata.py:326-365.
+
+`single_rank_plan` lays out what one CA server holds for a list of documents cut into
+shards when linear rank and attention rank are the same GPU: the task list (shard i of a
+document attends to the document's first i+1 shards, compute_metadata.py:404-448), the
+K/V shard entries with their main-copy mask and duplicate-gradient metadata (:202-219,
+277-323), and contiguous byte offsets for the q | k | v regions of each buffer.  The
+reference derives the same quantities for any number of ranks from planner output
+(_from_planner_output, :368-639); the multi-rank offset assignment is outside this build.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from .utils import exclusive_cumsum, prepend_zero_fn, size_pad_by_int4
+
+_TensorOrList = Union[Tensor, Sequence[Tensor]]
+
+
+def _dev(t: Tensor, dtype: torch.dtype, device) -> Tensor:
+    return t.to(device=device, dtype=dtype).contiguous()
+
+
+@dataclass
+class SeqLens:
+    send_seqlens: _TensorOrList
+    recv_seqlens: _TensorOrList
+
+    def get_slice(self, rank):
+        return SeqLens(self.send_seqlens[rank], self.recv_seqlens[rank])
+
+    def normalize(self, device="cuda"):
+        if isinstance(self.send_seqlens, Tensor):
+            return SeqLens(_dev(self.send_seqlens, torch.int64, device), _dev(self.recv_seqlens, torch.int64, device))
+        return SeqLens(tuple(_dev(t, torch.int64, device) for t in self.send_seqlens),
+                       tuple(_dev(t, torch.int64, device) for t in self.recv_seqlens))
+
+
+@dataclass
+class LogicalShape:
+    """Shapes used to allocate receive tensors; a KV send shape is (cp_degree, tokens, hidden)."""
+    send_shape: Union[torch.Size, Sequence[torch.Size]]
+    recv_shape: Union[torch.Size, Sequence[torch.Size]]
+
+    def get_slice(self, rank):
+        return LogicalShape(self.send_shape[rank], self.recv_shape[rank])
+
+
+@dataclass
+class DedupGradSumMetadata:
+    """A KV shard used by several query shards of a rank has several copies there; one copy
+    is sent forward, and the copies' gradients are summed into the main copy before one
+    gradient is sent back."""
+    num_copies: Tensor       # int32 [entries]
+    copy_start_id: Tensor    # int64 [entries, max_copies], token index of each duplicate
+    main_copy_mask: Tensor   # int8 [entries]
+
+    def normalize(self, device="cuda"):
+        return DedupGradSumMetadata(_dev(self.num_copies, torch.int32, device),
+                                    _dev(self.copy_start_id, torch.int64, device),
+                                    _dev(self.main_copy_mask, torch.int8, device))
+
+
+def get_attn_metadata(seqlens_q, seqlens_kv=None, get_packed_seq_params: bool = False):
+    """cu_seqlens / max_seqlen of a task list (one tensor) or of one list per rank."""
+    from .fused_comm_attn import PackedSeqParams
+    return_list = True
+    if seqlens_kv is None:
+        seqlens_kv = seqlens_q
+    if isinstance(seqlens_q, Tensor):
+        assert isinstance(seqlens_kv, Tensor)
+        seqlens_q, seqlens_kv = [seqlens_q], [seqlens_kv]
+        return_list = False
+    assert len(seqlens_kv) == len(seqlens_q)
+    world = []
+    for sq, skv in zip(seqlens_q, seqlens_kv):
+        assert sq.ndim == 1 and skv.shape == sq.shape
+        out = dict(cu_seqlens_q=prepend_zero_fn(sq.cumsum(dim=0)), cu_seqlens_kv=prepend_zero_fn(skv.cumsum(dim=0)),
+                   max_seqlen_q=sq.max().item(), max_seqlen_kv=skv.max().item())
+        if get_packed_seq_params:
+            out = PackedSeqParams(qkv_format="thd", **out)
+        world.append(out)
+    return world if return_list else world[0]
+
+
+@dataclass
+class SingleRankPlan:
+    """Everything one CA-server tick needs for `docs` (host tensors; `.to(device)` variants
+    are built by server_metas)."""
+    q_seqlens: Tensor            # int64 [tasks]  Lq of each task = its shard length
+    kv_seqlens: Tensor           # int64 [tasks]  Lk = document tokens up to the end of the shard
+    kv_entry_tokens: Tensor      # int64 [entries] K/V shard entries in task order (prefix shards per task)
+    kv_entry_shard: Tensor       # int64 [entries] index of the stored shard each entry reads
+    dedup: DedupGradSumMetadata
+    num_heads_q: int
+    num_heads_kv: int
+    head_dim: int
+    itemsize: int
+
+    @property
+    def num_q_tokens(self) -> int:
+        return int(self.q_seqlens.sum())
+
+    @property
+    def num_kv_tokens(self) -> int:
+        return int(self.kv_entry_tokens.sum())
+
+    # -- token sizes in bytes -------------------------------------------------------------
+    @property
+    def q_bytes(self) -> int:
+        return self.num_heads_q * self.head_dim * self.itemsize
+
+    @property
+    def k_bytes(self) -> int:
+        return self.num_heads_kv * self.head_dim * self.itemsize
+
+    @property
+    def out_lse_bytes(self) -> int:
+        """[out | lse fp32 per head | pad to 16] (attn_kernels/dispatch.py:209-221)."""
+        return size_pad_by_int4(self.q_bytes + self.num_heads_q * 4, 1)[0]
+
+    @property
+    def merged_q_bytes(self) -> int:
+        """[dO | O | lse | q | pad to 16] (attn_kernels/dispatch.py:138-158)."""
+        return size_pad_by_int4(3 * self.q_bytes + self.num_heads_q * 4, 1)[0]
+
+    def _regions(self, q_token_bytes: int) -> Tuple[Tensor, Tensor, Tensor, int]:
+        """Contiguous q | k | v regions, shards in order: (q offsets per task, k and v offsets per
+        stored shard, total bytes)."""
+        stored = self.stored_shard_tokens
+        q_off = exclusive_cumsum(self.q_seqlens * q_token_bytes)
+        base = int((self.q_seqlens * q_token_bytes).sum())
+        ksz = stored * self.k_bytes
+        k_off = base + exclusive_cumsum(ksz)
+        v_off = k_off + int(ksz.sum())
+        return q_off, k_off, v_off, base + 2 * int(ksz.sum())
+
+    @property
+    def stored_shard_tokens(self) -> Tensor:
+        """Tokens of each distinct K/V shard; equals q_seqlens because every shard is both a query
+        shard and a K/V shard of its document."""
+        return self.q_seqlens
+
+    def request_layout(self, backward: bool):
+        """(q offsets [tasks], k offsets [entries], v offsets [entries], bytes) of the receive
+        buffer; entries of one stored shard alias its single copy."""
+        q_off, k_off, v_off, total = self._regions(self.merged_q_bytes if backward else self.q_bytes)
+        return q_off, k_off[self.kv_entry_shard], v_off[self.kv_entry_shard], total
+
+    def reply_layout(self, backward: bool):
+        """Send buffer: forward [out|lse] per task; backward dq per task and dk, dv per stored
+        shard (entries that are not main copies keep their main's offset and are masked out)."""
+        if not backward:
+            off = exclusive_cumsum(self.q_seqlens * self.out_lse_bytes)
+            return off, None, None, int((self.q_seqlens * self.out_lse_bytes).sum())
+        q_off, k_off, v_off, total = self._regions(self.q_bytes)
+        return q_off, k_off[self.kv_entry_shard], v_off[self.kv_entry_shard], total
+
+
+def single_rank_plan(docs: Sequence[Sequence[int]], num_heads_q: int, num_heads_kv: int, head_dim: int = 128,
+                     itemsize: int = 2) -> SingleRankPlan:
+    """`docs[d]` = shard lengths tiling document d in order.  One task per shard."""
+    q_lens: List[int] = []
+    kv_lens: List[int] = []
+    entry_tokens: List[int] = []
+    entry_shard: List[int] = []
+    shard_base = 0
+    for doc in docs:
+        context = 0
+        for i, n in enumerate(doc):
+            if n <= 0:
+                raise ValueError("shard lengths must be positive")
+            context += n
+            q_lens.append(n)
+            kv_lens.append(context)
+            for j in range(i + 1):
+                entry_tokens.append(doc[j])
+                entry_shard.append(shard_base + j)
+        shard_base += len(doc)
+    entry_tokens_t = torch.tensor(entry_tokens, dtype=torch.int64)
+    entry_shard_t = torch.tensor(entry_shard, dtype=torch.int64)
+    starts = exclusive_cumsum(entry_tokens_t).tolist() if entry_tokens else []
+    first = {}
+    copies: List[List[int]] = [[] for _ in entry_tokens]
+    main_mask = [0] * len(entry_tokens)
+    for e, s in enumerate(entry_shard):
+        if s not in first:
+            first[s] = e
+            main_mask[e] = 1
+        else:
+            copies[first[s]].append(starts[e])
+    max_copies = max([len(c) for c in copies] + [1])
+    copy_start = torch.zeros((len(entry_tokens), max_copies), dtype=torch.int64)
+    for e, c in enumerate(copies):
+        if c:
+            copy_start[e, :len(c)] = torch.tensor(c, dtype=torch.int64)
+    dedup = DedupGradSumMetadata(torch.tensor([len(c) for c in copies], dtype=torch.int32), copy_start,
+                                 torch.tensor(main_mask, dtype=torch.int8))
+    return SingleRankPlan(torch.tensor(q_lens, dtype=torch.int64), torch.tensor(kv_lens, dtype=torch.int64),
+                          entry_tokens_t, entry_shard_t, dedup, num_heads_q, num_heads_kv, head_dim, itemsize)
+
+
+def server_metas(plan: SingleRankPlan, device="cuda"):
+    """(PackedSeqParams, ServerFwdMeta, ServerBwdMeta, buffer sizes) on `device` for one tick:
+    sizes = (fwd receive, fwd send, bwd receive, bwd send) bytes."""
+    from .fused_comm_attn import ServerBwdMeta, ServerFwdMeta
+    i64 = lambda t: _dev(t, torch.int64, device)
+    attn = get_attn_metadata(plan.q_seqlens, plan.kv_seqlens, get_packed_seq_params=True)
+    attn.cu_seqlens_q = _dev(attn.cu_seqlens_q, torch.int32, device)
+    attn.cu_seqlens_kv = _dev(attn.cu_seqlens_kv, torch.int32, device)
+    hq_d = plan.num_heads_q * plan.head_dim
+    hkv_d = plan.num_heads_kv * plan.head_dim
+    tq, tk = plan.num_q_tokens, plan.num_kv_tokens
+    fq, fk, fv, f_recv = plan.request_layout(False)
+    fo, _, _, f_send = plan.reply_layout(False)
+    fwd = ServerFwdMeta(i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(fq), i64(fk), i64(fv),
+                        i64(plan.q_seqlens), i64(fo), (tq, hq_d), (tk, hkv_d))
+    bq, bk, bv, b_recv = plan.request_layout(True)
+    gq, gk, gv, b_send = plan.reply_layout(True)
+    d = plan.dedup.normalize(device)
+    bwd = ServerBwdMeta(i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(bq), i64(bk), i64(bv),
+                        i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(gq), i64(gk), i64(gv),
+                        d.main_copy_mask, d.num_copies, d.copy_start_id, (tq, hq_d), (tq, plan.num_heads_q), (tk, hkv_d))
+    return attn, fwd, bwd, (f_recv, f_send, b_recv, b_send)

@@ -177,3 +177,67 @@ def test_grad_sum_matches_oracle_on_attention_gradients(cuda):
     got = data.to(cuda)
     pre_a2a_grad_acc(got, _dev(num_copies, cuda, torch.int32), _dev(starts, cuda, torch.int64), _dev(lens, cuda, torch.int64))
     assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+
+
+def test_server_tick_from_single_rank_plan(cuda):
+    """Two documents cut into shards; buffers laid out by metadata.single_rank_plan; the reply of the
+    backward tick, unpacked per stored shard, equals the whole-document gradients."""
+    from distca_amd import metadata
+    from distca_amd.fused_comm_attn import FlashAttnArgs, ca_server_backward, ca_server_forward
+    docs = [[130, 257, 64, 300], [90, 10]]
+    plan = metadata.single_rank_plan(docs, 8, 2)
+    fa_params, fmeta, bmeta, (f_recv, f_send, b_recv, b_send) = metadata.server_metas(plan, cuda)
+    fa_args = FlashAttnArgs(8, 2, 128)
+    T = plan.num_q_tokens
+    q, k, v, do = make_qkv(T, T, 8, 2, 128, 33)
+    as_bytes = lambda x: x.reshape(x.shape[0], -1).contiguous().view(torch.uint8).numpy()
+    stored = plan.stored_shard_tokens.numpy()
+    first_entry = [plan.kv_entry_shard.tolist().index(s) for s in range(len(stored))]
+
+    q_off, k_off, v_off, _ = plan.request_layout(False)
+    recv = np.zeros(f_recv, np.uint8)
+    fa2a.copy_non_cp(as_bytes(q), recv, q_off.numpy(), plan.q_seqlens.numpy())
+    fa2a.copy_non_cp(as_bytes(k), recv, k_off.numpy()[first_entry], stored)
+    fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
+    send = torch.zeros(f_send, dtype=torch.uint8, device=cuda)
+    print("plan forward", flush=True)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args)
+    torch.cuda.synchronize()
+    cu_doc = np.concatenate([[0], np.cumsum([sum(d) for d in docs])]).astype(np.int32)
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_doc, cu_doc)
+    assert_close_bf16(out.reshape(T, 8, 128), ref_out, "out")
+
+    # the linear side unpacks [out | lse] from the reply
+    reply = np.zeros((T, plan.out_lse_bytes), np.uint8)
+    fa2a.copy_non_cp(reply, send.cpu().numpy(), plan.reply_layout(False)[0].numpy(), plan.q_seqlens.numpy(), None, False)
+    assert np.array_equal(reply[:, :plan.q_bytes], as_bytes(out.cpu()))
+    lse_back = torch.from_numpy(reply[:, plan.q_bytes:plan.q_bytes + 32].copy()).view(torch.float32)   # [T, Hq]
+    assert torch.equal(lse_back, lse.T.cpu())
+
+    # backward request [dO | O | lse | q | pad]
+    merged = np.zeros((T, plan.merged_q_bytes), np.uint8)
+    c = 0
+    for part in (as_bytes(do), as_bytes(out.cpu()), reply[:, plan.q_bytes:plan.q_bytes + 32], as_bytes(q)):
+        merged[:, c:c + part.shape[1]] = part; c += part.shape[1]
+    q_off, k_off, v_off, _ = plan.request_layout(True)
+    recv = np.zeros(b_recv, np.uint8)
+    fa2a.copy_non_cp(merged, recv, q_off.numpy(), plan.q_seqlens.numpy())
+    fa2a.copy_non_cp(as_bytes(k), recv, k_off.numpy()[first_entry], stored)
+    fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
+    gsend = torch.zeros(b_send, dtype=torch.uint8, device=cuda)
+    print("plan backward", flush=True)
+    ca_server_backward(torch.from_numpy(recv).to(cuda), gsend, bmeta, fa_args, fa_params.cu_seqlens_q,
+                       fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
+    torch.cuda.synchronize()
+    gq_off, gk_off, gv_off, _ = plan.reply_layout(True)
+    g = gsend.cpu().numpy()
+    dq = np.zeros((T, plan.q_bytes), np.uint8); dk = np.zeros((T, plan.k_bytes), np.uint8); dv = np.zeros_like(dk)
+    fa2a.copy_non_cp(dq, g, gq_off.numpy(), plan.q_seqlens.numpy(), None, False)
+    fa2a.copy_non_cp(dk, g, gk_off.numpy()[first_entry], stored, None, False)
+    fa2a.copy_non_cp(dv, g, gv_off.numpy()[first_entry], stored, None, False)
+    tb = lambda a, h: torch.from_numpy(a).view(torch.bfloat16).reshape(T, h, 128)
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=out.cpu().reshape(T, 8, 128), softmax_lse=lse.cpu())
+    assert_close_bf16(tb(dq, 8), ref_dq, "dq")
+    # a stored shard's gradient is the bf16 sum of up to four per-task bf16 gradients: 4e-2 / 3e-3
+    assert_close_bf16(tb(dk, 2), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
+    assert_close_bf16(tb(dv, 2), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
