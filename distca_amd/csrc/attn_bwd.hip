@@ -11,20 +11,21 @@
 //
 //   1. bwd_prepare_kernel: per (token, head) row, scale*<dO, O> and lse*log2(e) -> workspace.
 //   2. ca_bwd_dkdv_kernel: one workgroup of 8 waves per (task, block of 128 keys, kv head),
-//      in the order of the backward tile schedule.  K and V of the block sit in LDS for the
-//      workgroup's life.  The query side (Q, dO and the two row statistics of every head of
+//      in the order of the backward tile schedule.  V of the block sits in LDS for the
+//      workgroup's life, K in registers (each wave's 32 keys as B operand).  The query side (Q, dO and the two row statistics of every head of
 //      the kv group, flattened into rows like the forward) is streamed in blocks of 32 rows
 //      from the first block the causal mask lets see these keys.  The waves form two groups of
 //      four; per iteration group 0 takes query block 2i and group 1 block 2i+1, so that every
 //      SIMD holds two waves at different points of the loop body.  In a group wave w owns
 //      keys 32w..32w+31:
-//        S = Q K^T, dP = dO V^T            A from the query tile, B from the K / V tiles (LDS)
+//        S = Q K^T, dP = dO V^T            A from the query tile, B = K registers / V tile (LDS)
 //        P = exp2(S*c - lse2), dS = P (dP*scale - delta*scale)          in registers
 //        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
 //                                          B = the accumulator registers converted to bf16
-//      Query tiles arrive one iteration ahead through LDS-direct global loads, one 256-byte
-//      row per instruction so the tile keeps its padded pitch.  After the loop group 1 hands
-//      its partial sums to group 0 through LDS.
+//      Query tiles arrive one iteration ahead through LDS-direct global loads, four 256-byte
+//      rows per instruction; the tile has unpadded rows whose 16-byte chunks are swizzled
+//      (tile_swz), which serves both read shapes without bank conflicts.  After the loop
+//      group 1 hands its partial sums to group 0 through LDS.
 //   3. ca_bwd_dq_kernel: one workgroup of 4 waves per (task, block of 128 flattened query
 //      rows, kv head), in the order of the forward tile schedule; the mirror image of the
 //      forward kernel.  Q and dO stay in registers as B operands, K/V tiles of 64 keys are
@@ -55,8 +56,9 @@ constexpr int kBM = kBwdRows;  // 32 flattened query rows per block
 constexpr int kKsOff = 0;
 constexpr int kVsOff = kKsOff + kBN * kPitch;
 constexpr int kTileOff = kVsOff + kBN * kPitch;
-constexpr int kTileQ = 0, kTileDO = kBM * kPitch;
-constexpr int kTileBytes = 2 * kBM * kPitch;      // Q + dO of one block
+constexpr int kTileRow = 256;                     // query-side tiles: unpadded rows, swizzled chunks (tile_swz)
+constexpr int kTileQ = 0, kTileDO = kBM * kTileRow;
+constexpr int kTileBytes = 2 * kBM * kTileRow;    // Q + dO of one block
 constexpr int kStatOff = kTileOff + 4 * kTileBytes;  // tiles: [stage 0/1][group 0/1]
 constexpr int kStatBytes = 3 * kBM * 4;           // per (stage, group): lse2, dscaled, lim
 constexpr int kBwdLds = kStatOff + 4 * kStatBytes;
@@ -73,6 +75,7 @@ struct BwdArgs {
   const int32_t *sched;
   int32_t sched_items_off;
   int32_t hq, hkv, group, total_q;
+  uint32_t group_magic;  // ceil(2^32 / group), 0 when group == 1: n / group == umulhi(n, magic) for n * group < 2^32
   int32_t causal;
   float scale;
 };
@@ -143,46 +146,58 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
 
   const int64_t qbase = ((int64_t)q0 * a.hq + kvh * G) * kHeadDim;  // element offset of (token q0, first head of the group)
 
-  // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block
+  // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block.
+  // Rows past the task (and a group's last block when it does not exist) are clamped to the
+  // task's last row so that the loads stay in bounds, and marked by lim = -1 (every key masked).
+  auto div_group = [&](int n) { return a.group_magic ? (int)__umulhi((uint32_t)n, a.group_magic) : n; };
   auto issue_tile = [&](int stage, int mbx) {
     const int tile = kTileOff + (stage * 2 + grp) * kTileBytes;
     const int stat = kStatOff + (stage * 2 + grp) * kStatBytes;
-    // lanes 0..7 work out one row each; rows past the task are clamped to its last row so that
-    // the loads stay in bounds, and marked by lim = -1 (every key masked)
-    const int rl = kbw * 8 + (lane & 7);
-    const int rho = mbx * kBM + rl;
-    const bool ok = rho < nrows && mbx >= mb0;  // a group's last block may not exist
-    const int rc = ok ? rho : nrows - 1;
-    const int tok = rc / G;
-    const int hg = rc - tok * G;
-    const int ro = tok * a.hq + hg;
-    if (lane < 8) {
-      int lm = a.causal ? tok + shift : lk - 1;
-      if (lm > lk - 1) lm = lk - 1;
-      reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
-      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
-      lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
-      lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int ro_i = __builtin_amdgcn_readlane(ro, i);
-      const __bf16 *qrow = a.q + qbase + (int64_t)ro_i * kHeadDim;
-      const __bf16 *dorow = a.dout + qbase + (int64_t)ro_i * kHeadDim;
-      const uint32_t dst = lds0 + tile + (kbw * 8 + i) * kPitch;
-      if (lane < 16) {
-        lds_direct_load16(qrow, lane * 16, dst + kTileQ);
-        lds_direct_load16(dorow, lane * 16, dst + kTileDO);
+    const bool blk_ok = mbx >= mb0;
+    {  // row statistics: lanes 0..7 take one row each
+      const int rl = kbw * 8 + (lane & 7);
+      const int rho = mbx * kBM + rl;
+      const bool ok = blk_ok && rho < nrows;
+      const int rc = ok ? rho : nrows - 1;
+      const int tok = div_group(rc);
+      const int hg = rc - tok * G;
+      if (lane < 8) {
+        int lm = a.causal ? tok + shift : lk - 1;
+        if (lm > lk - 1) lm = lk - 1;
+        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
+        const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
+        lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
+        lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
       }
+    }
+    // Q and dO: one instruction fills four rows; lane p brings the chunk that belongs at chunk
+    // position p%16 of row p/16
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int rl = kbw * 8 + 4 * i + (lane >> 4);
+      const int rho = mbx * kBM + rl;
+      const bool ok = blk_ok && rho < nrows;
+      const int rc = ok ? rho : nrows - 1;
+      const int tok = div_group(rc);
+      const int hg = rc - tok * G;
+      const int chunk = (lane & 15) ^ tile_swz(rl);
+      const int64_t eo = qbase + (int64_t)(tok * a.hq + hg) * kHeadDim + chunk * 8;
+      const uint32_t dst = lds0 + tile + (kbw * 8 + 4 * i) * kTileRow;
+      lds_direct_load16_ptr(a.q + eo, dst + kTileQ);
+      lds_direct_load16_ptr(a.dout + eo, dst + kTileDO);
     }
   };
 
   const float c = a.scale * kLog2e;
   // tile-independent LDS offsets
-  const int a_rd = l32 * kPitch + 16 * g;                // A operand rows, + 32*s
-  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;   // B operand rows of K / V, + 32*s
-  const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // transposed A
+  const int a_rd = l32 * kTileRow + ((g ^ tile_swz(l32)) << 4);  // A operand rows of the query tile, ^ 32*s
+  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;           // B operand rows of K / V, + 32*s
+  // transposed A operand: lane points at (row 4g + i4 [+8 hi +16 (j>>2)], chunk 8 b4 + h1 [+2 (j&3)], half lane&1);
+  // tile_swz of that row is (i4<<1) | (g<<3) | hi
+  const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
+  const int t_rd = (4 * g + i4) * kTileRow + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*(j&3) ^ 16*hi
 
+  bf16x8 kreg[8];  // this wave's 32 keys as B operand of S = Q K^T, all 8 steps over d
   f32x16 sacc, dpacc;
   // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
   auto phase_a = [&](int stage) {
@@ -193,32 +208,32 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       dpacc[r] = 0.f;
     }
     // operands of step s+1 are requested before the MFMAs of step s are issued
-    bf16x8 qa[2], kb[2], da[2], vb[2];
+    constexpr int kDa = 2;  // operand fetch distance in MFMA steps
+    bf16x8 qa[kDa], da[kDa], vb[kDa];
     auto load_a = [&](int s, int buf) {
-      qa[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + a_rd + 32 * s);
-      kb[buf] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
-      da[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + a_rd + 32 * s);
+      const int ao = a_rd ^ (s << 5);
+      qa[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + ao);
+      da[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + ao);
       vb[buf] = *reinterpret_cast<const bf16x8 *>(lds + kVsOff + b_rd + 32 * s);
     };
-    load_a(0, 0);
-    load_a(1, 1);
+#pragma unroll
+    for (int s = 0; s < kDa; ++s) load_a(s, s);
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       __builtin_amdgcn_sched_barrier(0);
-      sacc = mfma32(qa[s & 1], kb[s & 1], sacc);
-      dpacc = mfma32(da[s & 1], vb[s & 1], dpacc);
+      sacc = mfma32(qa[s % kDa], kreg[s], sacc);
+      dpacc = mfma32(da[s % kDa], vb[s % kDa], dpacc);
       __builtin_amdgcn_sched_barrier(0);
-      if (s + 2 < 8) load_a(s + 2, s & 1);
+      if (s + kDa < 8) load_a(s + kDa, s % kDa);
     }
   };
-  // ---- phase B (VALU): P and dS in registers; phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
-  auto phase_bc = [&](int stage) {
-    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+  // ---- phase B (VALU): P and dS, converted to bf16 B operands
+  bf16x8 pb[2], dsb[2];
+  auto phase_b = [&](int stage) {
     const uint8_t *stat = lds + kStatOff + (stage * 2 + grp) * kStatBytes;
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
     const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
     const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
-    bf16x8 pb[2], dsb[2];
 #pragma unroll
     for (int cq = 0; cq < 4; ++cq) {
       const int qr = 8 * cq + 4 * g;
@@ -242,23 +257,29 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
       dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
     }
-    bf16x4 ct[2][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
+  };
+  // ---- phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
+  auto phase_c = [&](int stage) {
+    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+    constexpr int kDc = 2;  // operand fetch distance in MFMA steps
+    bf16x4 ct[kDc][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
     auto load_c = [&](int j, int buf) {
-      const int off = 16 * (j >> 2) * kPitch + t_rd + 32 * (j & 3);
-      ct[buf][0] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off));
-      ct[buf][1] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + off + 8 * kPitch));
-      ct[buf][2] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off));
-      ct[buf][3] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + off + 8 * kPitch));
+      const int lo = (16 * (j >> 2)) * kTileRow + (t_rd ^ ((j & 3) << 5));
+      const int hi = (16 * (j >> 2) + 8) * kTileRow + (t_rd ^ ((j & 3) << 5) ^ 16);
+      ct[buf][0] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + lo));
+      ct[buf][1] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + hi));
+      ct[buf][2] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + lo));
+      ct[buf][3] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + hi));
     };
-    load_c(0, 0);
-    load_c(1, 1);
+#pragma unroll
+    for (int j = 0; j < kDc; ++j) load_c(j, j);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       __builtin_amdgcn_sched_barrier(0);
-      dvacc[j & 3] = mfma32(cat4(ct[j & 1][0], ct[j & 1][1]), pb[j >> 2], dvacc[j & 3]);
-      dkacc[j & 3] = mfma32(cat4(ct[j & 1][2], ct[j & 1][3]), dsb[j >> 2], dkacc[j & 3]);
+      dvacc[j & 3] = mfma32(cat4(ct[j % kDc][0], ct[j % kDc][1]), pb[j >> 2], dvacc[j & 3]);
+      dkacc[j & 3] = mfma32(cat4(ct[j % kDc][2], ct[j % kDc][3]), dsb[j >> 2], dkacc[j & 3]);
       __builtin_amdgcn_sched_barrier(0);
-      if (j + 2 < 8) load_c(j + 2, j & 1);
+      if (j + kDc < 8) load_c(j + kDc, j % kDc);
     }
   };
 
@@ -266,8 +287,10 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // period group 0 is in its MFMA-only phase A while group 1 starts with the VALU-heavy
   // phase B; after the second barrier the roles swap.  A SIMD holds one wave of each
   // group, so its MFMA pipe and its VALU are busy at the same time instead of by turns.
-  //   period p:  [barrier 1]  g0: A(p)          g1: B,C(p-1)
-  //              [barrier 2]  g0: B,C(p)        g1: A(p)
+  //   period p:  [barrier 1]  g0: fetch(p+1), A(p)   g1: B,C(p-1)
+  //              [barrier 2]  g0: B,C(p)             g1: fetch(p+1), A(p)
+  // (Moving B in front of the second barrier, which evens out the instruction counts of the two
+  // halves, measured 14 % slower: phases A and C both live on LDS reads and then run together.)
   // A group's tile p+1 is requested right after the barrier that retires tile p-1 and is
   // waited for before the same barrier one period later.
   // Each group has its own copy of the loop (every wave still passes the same 2*(niter+1)
@@ -276,6 +299,9 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // same time (neighbouring key blocks of one document, by the schedule) then read the same
   // query rows at the same time and find them in their XCD's L2.
   if (niter > 0) issue_tile(0, nmb - 1 - grp);
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
   if (grp == 0) {
     for (int p = 0; p < niter; ++p) {
       const int stage = p & 1;
@@ -284,7 +310,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 1 - 2 * (p + 1));
       phase_a(stage);
       __syncthreads();
-      phase_bc(stage);
+      phase_b(stage);
+      phase_c(stage);
     }
     __syncthreads();
     __syncthreads();
@@ -297,7 +324,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 2 - 2 * (p + 1));
       phase_a(stage);
       __syncthreads();
-      phase_bc(stage);
+      phase_b(stage);
+      phase_c(stage);
     }
     __syncthreads();
   }
@@ -694,6 +722,9 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
+  a.group_magic = a.group == 1 ? 0u : (uint32_t)(((1ull << 32) + a.group - 1) / a.group);
+  if ((uint64_t)p->max_seqlen_q * a.group * a.group >= (1ull << 32))
+    return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: max_seqlen_q * (Hq/Hkv)^2 must stay below 2^32");
 
   static bool attr_set = false;
   if (!attr_set) {

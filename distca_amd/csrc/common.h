@@ -68,10 +68,21 @@ __device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t vo
   const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbu), "s"(uniform32(lds_base)) : "memory");
 }
+// 16 bytes per lane from a per-lane pointer; lane L's data lands at lds_base + 16*L.
+__device__ __forceinline__ void lds_direct_load16_ptr(const void *gptr_lane, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
+}
 __device__ __forceinline__ void lds_direct_load4(const void *gptr_lane, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
 }
 __device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Swizzle of a row-major LDS tile with 256-byte rows (16 chunks of 16 bytes, no padding):
+// chunk c of row r is stored at chunk position c ^ tile_swz(r).  With it both read shapes of
+// the MFMA operands are free of bank conflicts (128-bit reads of one chunk column over 32 rows,
+// and the transposing 64-bit reads over 4-row x 32-byte patches), and a row keeps its 256
+// contiguous bytes, so LDS-direct loads can fill four rows per instruction.
+__device__ __forceinline__ int tile_swz(int r) { return ((r & 3) << 1) | ((r & 4) << 1) | ((r >> 3) & 1); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
