@@ -641,8 +641,8 @@ struct BwdWorkspace {
 BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias) {
   BwdWorkspace w;
   int64_t o = 0;
-  w.sched_kv = o; o += align_up(sched_bytes(p->num_tasks, bwd_max_items(p)), 256);
-  w.sched_q = o; o += align_up(sched_bytes(p->num_tasks, fwd_max_items(p)), 256);
+  w.sched_kv = o; o += sched_region_bytes(p->num_tasks, bwd_max_items(p));
+  w.sched_q = o; o += sched_region_bytes(p->num_tasks, dq_max_items(p));
   w.delta = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.lse2 = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.dk_acc = o; if (alias) o += align_up((int64_t)p->total_k * p->num_heads_kv * kHeadDim * 4, 256);
@@ -752,8 +752,8 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   }
   // ---- dQ: one workgroup per (task, block of query rows, kv head)
   {
-    const SchedGeom geom = fwd_geom(p);
-    const int64_t max_items = fwd_max_items(p);
+    const SchedGeom geom = dq_geom(p);
+    const int64_t max_items = dq_max_items(p);
     rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
     if (rc) return rc;
     const int64_t grid = max_items * p->num_heads_kv;

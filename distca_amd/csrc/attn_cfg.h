@@ -9,15 +9,20 @@
 namespace distca {
 
 constexpr int kHeadDim = 128;
-constexpr int kWaves = 4;  // waves per workgroup in every attention kernel
+constexpr int kWaves = 4;  // waves per workgroup of the dQ kernel
 
 // Forward and dQ kernels: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles
-// of 64 keys.  One sub-tile keeps a wave under 256 registers, so two workgroups share a CU.
+// of 64 keys.  One sub-tile keeps a wave under 256 registers, so a compute unit holds eight waves.
 #ifndef DISTCA_FWD_MSUB
 #define DISTCA_FWD_MSUB 1
 #endif
+#ifndef DISTCA_FWD_WAVES
+#define DISTCA_FWD_WAVES 8
+#endif
 constexpr int kFwdMsub = DISTCA_FWD_MSUB;
-constexpr int kFwdRows = kWaves * 32 * kFwdMsub;
+constexpr int kFwdWaves = DISTCA_FWD_WAVES;  // waves per workgroup of the forward kernel
+constexpr int kFwdRows = kFwdWaves * 32 * kFwdMsub;
+constexpr int kDqRows = kWaves * 32 * kFwdMsub;
 constexpr int kFwdKV = 64;
 
 // Backward: a workgroup owns 128 keys (four waves of 32, in two copies that take alternate
@@ -47,6 +52,11 @@ inline SchedGeom fwd_geom(const distca_ca_params *p) {
   g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_k / kFwdKV + 1);
   return g;
 }
+inline SchedGeom dq_geom(const distca_ca_params *p) {
+  SchedGeom g = fwd_geom(p);
+  g.rows_per_block = kDqRows;
+  return g;
+}
 inline SchedGeom bwd_geom(const distca_ca_params *p) {
   SchedGeom g;
   g.rows_per_block = kBwdRows;
@@ -60,6 +70,10 @@ inline SchedGeom bwd_geom(const distca_ca_params *p) {
 inline int64_t fwd_max_items(const distca_ca_params *p) {
   const int64_t group = p->num_heads_q / p->num_heads_kv;
   return (int64_t)p->total_q * group / kFwdRows + p->num_tasks + 1;
+}
+inline int64_t dq_max_items(const distca_ca_params *p) {
+  const int64_t group = p->num_heads_q / p->num_heads_kv;
+  return (int64_t)p->total_q * group / kDqRows + p->num_tasks + 1;
 }
 inline int64_t bwd_max_items(const distca_ca_params *p) {
   // sum over tasks of ceil(Lk / kBwdKV); sum of Lk may exceed total_k when prefixes alias,

@@ -5,10 +5,12 @@
 //
 // Work decomposition.  The G = Hq/Hkv query heads that share a kv head are flattened with
 // the tokens into one row axis: row R of a task = (token R / G, head R % G), so one K/V
-// tile in LDS serves all heads of its group.  A workgroup (4 waves) owns kRows consecutive
+// tile in LDS serves all heads of its group.  A workgroup (8 waves) owns kRows consecutive
 // flattened rows of one task and one kv head and streams that task's visible KV prefix in
 // tiles of 64 keys; tiles entirely above the diagonal are never visited and only tiles
-// that straddle it are masked.
+// that straddle it are masked.  With 8 waves a workgroup covers 256 rows per K/V tile it pulls
+// through the vector memory unit, whose throughput (about 64 bytes per clock per compute unit)
+// is what a 128-row workgroup ran into.
 //
 // Per wave: MSUB sub-tiles of 32 rows.  Scores are produced transposed, S^T = K Q^T, so a
 // lane holds one query row (column lane%32) and 16 keys per 32x32 block: the online-softmax
@@ -16,6 +18,12 @@
 // registers are, after conversion to bf16, already laid out as the B operand of
 // O^T += V^T P^T.  Q stays in registers for the whole KV loop; K is read from LDS row-major
 // (16-byte reads), V through the transposing LDS read.
+//
+// K/V tiles go from global memory straight into LDS (LDS-direct loads, four 256-byte rows per
+// instruction, rows unpadded with swizzled 16-byte chunks, see tile_swz).  The eight load
+// instructions a wave contributes to the next tile are issued one at a time between the MFMAs
+// of the current tile's S phase: issued in one burst after the barrier, every wave of the
+// compute unit queues at the vector memory unit at the same moment and the MFMA pipe idles.
 #include "api_util.h"
 #include "attn_cfg.h"
 #include "common.h"
@@ -23,10 +31,9 @@
 namespace distca {
 namespace {
 
-constexpr int kKPitch = 272;  // bytes per K row in LDS (256 + 16: rows shift by 4 banks)
-constexpr int kVPitch = 288;  // bytes per V row in LDS (256 + 32: 4 rows x 32 B tile the banks)
-constexpr int kKTile = kFwdKV * kKPitch;
-constexpr int kVTile = kFwdKV * kVPitch;
+constexpr int kRowB = 256;    // bytes per K or V row in LDS (unpadded; chunk c of row r sits at c ^ tile_swz(r))
+constexpr int kKTile = kFwdKV * kRowB;
+constexpr int kVTile = kFwdKV * kRowB;
 constexpr int kStage = kKTile + kVTile;
 constexpr int kFwdLds = 2 * kStage;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -38,6 +45,7 @@ struct FwdArgs {
   float *lse;
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;  // schedule workspace
+  const void *zero_row;  // 256 zero bytes: source of tile rows past the end of the prefix
   int32_t sched_items_off;  // int32 offset of the item array
   int32_t hq, hkv, group, total_q;
   int32_t causal;
@@ -45,7 +53,7 @@ struct FwdArgs {
 };
 
 template <int MSUB>
-__global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
+__global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   const int item = blockIdx.x / a.hkv;
@@ -63,7 +71,7 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  constexpr int kRows = kWaves * 32 * MSUB;
+  constexpr int kRows = kFwdWaves * 32 * MSUB;
   const int row_wg = mblk * kRows;
   const int nrows = lq * G;
 
@@ -114,35 +122,26 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
     }
   }
 
-  // ---- K/V tile staging: 64 rows x 16 chunks of 16 B, 4 chunks per thread
-  const int ld_col = tid & 15;  // 16-byte chunk within the row
-  const int ld_row = tid >> 4;  // + 16*i
+  // ---- K/V tile fetch: wave w brings rows 16w .. 16w+15 of the K tile and of the V tile, four
+  // rows per instruction; lane p fetches the chunk that belongs at chunk position p%16 of row p/16
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
-  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
-  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
-  u32x4 kreg[4], vreg[4];
-  auto load_tile = [&](int j) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = j * kFwdKV + ld_row + 16 * i;
-      if (key < lk) {
-        kreg[i] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)key * kv_stride);
-        vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + (int64_t)key * kv_stride);
-      } else {
-        kreg[i] = u32x4{0, 0, 0, 0};
-        vreg[i] = u32x4{0, 0, 0, 0};
-      }
-    }
-  };
-  auto store_tile = [&](int stage) {
-    uint8_t *kt = lds + stage * kStage;
-    uint8_t *vt = kt + kKTile;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = ld_row + 16 * i;
-      *reinterpret_cast<u32x4 *>(kt + r * kKPitch + ld_col * 16) = kreg[i];
-      *reinterpret_cast<u32x4 *>(vt + r * kVPitch + ld_col * 16) = vreg[i];
-    }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
+  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  // a wave brings kRowsW rows of the K tile and of the V tile: instructions 0 .. kLdW/2-1 fetch K
+  // rows kRowsW*w + 4i .. +3, the other half the same rows of V
+  constexpr int kRowsW = kFwdKV / kFwdWaves, kLdW = 2 * (kRowsW / 4);
+  auto issue_kv = [&](int j, int stage, int i) {
+    const bool is_k = i < kLdW / 2;
+    const int ii = is_k ? i : i - kLdW / 2;
+    const int r = kRowsW * uwave + 4 * ii + (lane >> 4);
+    const int key = j * kFwdKV + r;
+    const int chunk = (lane & 15) ^ tile_swz(r);
+    const __bf16 *src = (is_k ? kbase : vbase) + (int64_t)key * kv_stride;
+    if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
+    const uint32_t dst = lds0 + stage * kStage + (is_k ? 0 : kKTile) + (kRowsW * uwave + 4 * ii) * kRowB;
+    lds_direct_load16_ptr(src + chunk * 8, dst);
   };
 
   // ---- accumulators
@@ -160,13 +159,17 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
   const float c = a.scale * kLog2e;
 
   // LDS read offsets (bytes) that do not depend on the tile
-  const int k_rd = l32 * kKPitch + 16 * g;                                            // + kb*32*kKPitch + 32*s
-  const int v_rd = (4 * g + ((lane & 15) >> 2)) * kVPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // + (16t+8h)*kVPitch + 32*db
+  const int k_rd = l32 * kRowB + ((g ^ tile_swz(l32)) << 4);  // + kb*32*kRowB, ^ 32*s
+  // transposed V operand: lane points at (key 4g + i4 [+8 hi +16 t], chunk 8 b4 + h1 [+2 db], half lane&1);
+  // tile_swz of that row is (i4<<1) | (g<<3) | hi
+  const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
+  const int v_rd = (4 * g + i4) * kRowB + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*db ^ 16*hi
 
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
+#pragma unroll
+    for (int i = 0; i < kLdW; ++i) issue_kv(0, 0, i);
   }
+  wait_vm0();
   __syncthreads();
 
   for (int j = 0; j < ntiles; ++j) {
@@ -174,7 +177,6 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
     const uint8_t *kt = lds + stage * kStage;
     const uint8_t *vt = kt + kKTile;
     const bool has_next = j + 1 < ntiles;
-    if (has_next) load_tile(j + 1);
 
     const int key0 = j * kFwdKV;
     const bool active = wave_live && key0 <= lim_last;
@@ -188,14 +190,25 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) sacc[m][kb][r] = 0.f;
+      // K fragments are requested kPf steps before the MFMAs that use them
+      constexpr int kPf = 2;
+      bf16x8 kf[kPf][2];
+      auto load_k = [&](int s, int buf) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kRowB + (k_rd ^ (s << 5)));
+      };
+#pragma unroll
+      for (int s = 0; s < kPf; ++s) load_k(s, s);
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(kt + k_rd + kb * 32 * kKPitch + 32 * s);
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int m = 0; m < MSUB; ++m) sacc[m][kb] = mfma32(kf, qf[m][s], sacc[m][kb]);
-        }
+          for (int m = 0; m < MSUB; ++m) sacc[m][kb] = mfma32(kf[s % kPf][kb], qf[m][s], sacc[m][kb]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + kPf < 8) load_k(s + kPf, s % kPf);
+        if (has_next && s < kLdW) issue_kv(j + 1, stage ^ 1, s);  // next tile, one instruction per step
       }
       // ---- mask the tiles that straddle the diagonal or the end of the prefix
       if (key0 + kFwdKV - 1 > lim_first) {
@@ -248,25 +261,34 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_fwd_kernel(FwdArg
         }
       }
     }
-    // ---- next tile into the other LDS stage (its last readers finished before the
-    //      barrier that ended the previous iteration)
-    if (has_next) store_tile(stage ^ 1);
+    // a wave with nothing to compute in this tile still fetches its share of the next one (the
+    // other LDS stage: its last readers finished before the barrier that ended the previous iteration)
+    if (!active && has_next) {
+#pragma unroll
+      for (int i = 0; i < kLdW; ++i) issue_kv(j + 1, stage ^ 1, i);
+    }
 
     if (active) {
       // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
+      constexpr int kPfV = 4;  // V^T fragments are requested four MFMAs ahead
+      bf16x4 vf[kPfV][2];
+      auto load_v = [&](int u, int buf) {  // u = 4*t + db
+        const uint8_t *vp = vt + 16 * (u >> 2) * kRowB;
+        vf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(vp + (v_rd ^ ((u & 3) << 5))));
+        vf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kRowB + (v_rd ^ ((u & 3) << 5) ^ 16)));
+      };
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int u = 0; u < kPfV; ++u) load_v(u, u);
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const uint8_t *vp = vt + v_rd + 16 * t * kVPitch + 32 * db;
-          const bf16x4 lo = lds_read_tr((const DISTCA_LDS void *)vp);
-          const bf16x4 hi = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kVPitch));
-          const bf16x8 vf = cat4(lo, hi);
+      for (int u = 0; u < 16; ++u) {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int m = 0; m < MSUB; ++m) oacc[m][db] = mfma32(vf, pf[m][t], oacc[m][db]);
-        }
+        for (int m = 0; m < MSUB; ++m) oacc[m][u & 3] = mfma32(cat4(vf[u % kPfV][0], vf[u % kPfV][1]), pf[m][u >> 2], oacc[m][u & 3]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u + kPfV < 16) load_v(u + kPfV, u % kPfV);
       }
     }
+    wait_vm0();
     __syncthreads();
   }
 
@@ -305,7 +327,7 @@ extern "C" int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p) {
   if (!p) return fail(DISTCA_E_INVALID, "fwd_workspace_bytes: null params");
   int rc = validate_params(p);
   if (rc) return rc;
-  return align_up(sched_bytes(p->num_tasks, fwd_max_items(p)), 256);
+  return sched_region_bytes(p->num_tasks, fwd_max_items(p));
 }
 
 extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
@@ -331,6 +353,7 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
   a.out = (__bf16 *)out; a.lse = lse;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
   a.sched = (const int32_t *)workspace;
+  a.zero_row = (const uint8_t *)workspace + sched_zero_row_off(p->num_tasks, max_items);
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
@@ -344,7 +367,7 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);
-    hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kFwdLds, s, a);
+    hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
   }
   return check_launch("ca_fwd");
 }

@@ -82,5 +82,15 @@ DISTCA_HD int64_t sched_header_ints(int32_t num_tasks) { return ((int64_t)4 + nu
 DISTCA_HD int64_t sched_bytes(int32_t num_tasks, int64_t max_items) {
   return (sched_header_ints(num_tasks) + 4 * max_items) * (int64_t)sizeof(int32_t);
 }
+// A schedule region ends with 256 zero bytes, written by the builder: the attention kernels
+// point the tile loads of rows that do not exist (past the end of a task) at them, so that such
+// rows are finite whatever the neighbouring memory holds.
+constexpr int64_t kZeroRowBytes = 256;
+DISTCA_HD int64_t sched_zero_row_off(int32_t num_tasks, int64_t max_items) {
+  return (sched_bytes(num_tasks, max_items) + 255) / 256 * 256;
+}
+DISTCA_HD int64_t sched_region_bytes(int32_t num_tasks, int64_t max_items) {
+  return sched_zero_row_off(num_tasks, max_items) + kZeroRowBytes;
+}
 
 }  // namespace distca
