@@ -73,6 +73,7 @@ struct BwdArgs {
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;
+  const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
   int32_t sched_items_off;
   int32_t hq, hkv, group, total_q;
   uint32_t group_magic;  // ceil(2^32 / group), 0 when group == 1: n / group == umulhi(n, magic) for n * group < 2^32
@@ -382,11 +383,13 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
 // dQ
 // ------------------------------------------------------------------------------------------
 constexpr int kDqKV = kFwdKV;  // 64 keys per tile
-constexpr int kDqStage = 2 * kDqKV * kPitch;  // K tile + V tile
+constexpr int kDqRowB = 256;                   // unpadded rows, chunks swizzled by tile_swz
+constexpr int kDqTile = kDqKV * kDqRowB;
+constexpr int kDqStage = 2 * kDqTile;          // K tile + V tile
 constexpr int kDqLds = 2 * kDqStage;
 
 template <int MSUB>
-__global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(BwdArgs a) {
+__global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) void ca_bwd_dq_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   const int item = blockIdx.x / a.hkv;
@@ -458,34 +461,24 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(Bwd
     if (lim_last > lk - 1) lim_last = lk - 1;
   }
 
-  // ---- K/V tile staging: 64 rows x 16 chunks of 16 B, 4 chunks per thread and tensor
-  const int ld_col = tid & 15, ld_row = tid >> 4;
+  // ---- K/V tile fetch by LDS-direct loads, as in the forward kernel: a wave brings kRowsW rows of
+  // the K tile and of the V tile, four rows per instruction
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
-  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
-  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim + ld_col * 8;
-  u32x4 kreg[4], vreg[4];
-  auto load_tile = [&](int j) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = j * kDqKV + ld_row + 16 * i;
-      if (key < lk) {
-        kreg[i] = *reinterpret_cast<const u32x4 *>(kbase + (int64_t)key * kv_stride);
-        vreg[i] = *reinterpret_cast<const u32x4 *>(vbase + (int64_t)key * kv_stride);
-      } else {
-        kreg[i] = u32x4{0, 0, 0, 0};
-        vreg[i] = u32x4{0, 0, 0, 0};
-      }
-    }
-  };
-  auto store_tile = [&](int stage) {
-    uint8_t *kt = lds + stage * kDqStage;
-    uint8_t *vt = kt + kDqKV * kPitch;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = ld_row + 16 * i;
-      *reinterpret_cast<u32x4 *>(kt + r * kPitch + ld_col * 16) = kreg[i];
-      *reinterpret_cast<u32x4 *>(vt + r * kPitch + ld_col * 16) = vreg[i];
-    }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
+  const int uwave = __builtin_amdgcn_readfirstlane(wave);
+  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  constexpr int kRowsW = kDqKV / kWaves, kLdW = 2 * (kRowsW / 4);
+  auto issue_kv = [&](int j, int stage, int i) {
+    const bool is_k = i < kLdW / 2;
+    const int ii = is_k ? i : i - kLdW / 2;
+    const int r = kRowsW * uwave + 4 * ii + (lane >> 4);
+    const int key = j * kDqKV + r;
+    const int chunk = (lane & 15) ^ tile_swz(r);
+    const __bf16 *src = (is_k ? kbase : vbase) + (int64_t)key * kv_stride;
+    if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
+    const uint32_t dst = lds0 + stage * kDqStage + (is_k ? 0 : kDqTile) + (kRowsW * uwave + 4 * ii) * kDqRowB;
+    lds_direct_load16_ptr(src + chunk * 8, dst);
   };
 
   f32x16 dqacc[MSUB][4];
@@ -496,21 +489,23 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(Bwd
 #pragma unroll
       for (int r = 0; r < 16; ++r) dqacc[m][db][r] = 0.f;
   const float c = a.scale * kLog2e;
-  const int k_rd = l32 * kPitch + 16 * g;                                                                // + kb*32*kPitch + 32*s
-  const int t_rd = (4 * g + ((lane & 15) >> 2)) * kPitch + (64 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;  // + (16t+8h)*kPitch + 32*db
+  const int k_rd = l32 * kDqRowB + ((g ^ tile_swz(l32)) << 4);  // + kb*32*kDqRowB, ^ 32*s
+  // transposed K operand: lane points at (key 4g + i4 [+8 hi +16 t], chunk 8 b4 + h1 [+2 db], half lane&1)
+  const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
+  const int t_rd = (4 * g + i4) * kDqRowB + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*db ^ 16*hi
 
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
+#pragma unroll
+    for (int i = 0; i < kLdW; ++i) issue_kv(0, 0, i);
   }
+  wait_vm0();
   __syncthreads();
 
   for (int j = 0; j < ntiles; ++j) {
     const int stage = j & 1;
     const uint8_t *kt = lds + stage * kDqStage;
-    const uint8_t *vt = kt + kDqKV * kPitch;
+    const uint8_t *vt = kt + kDqTile;
     const bool has_next = j + 1 < ntiles;
-    if (has_next) load_tile(j + 1);
 
     const int key0 = j * kDqKV;
     const bool active = wave_live && key0 <= lim_last;
@@ -526,18 +521,32 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(Bwd
             sacc[m][kb][r] = 0.f;
             dpacc[m][kb][r] = 0.f;
           }
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
+      // operand fragments are requested kPf steps before the MFMAs that use them; the next tile's
+      // loads go out one instruction per step
+      constexpr int kPf = 1;
+      bf16x8 kf[kPf][2], vf[kPf][2];
+      auto load_kv = [&](int s, int buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(kt + k_rd + kb * 32 * kPitch + 32 * s);
-          const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(vt + k_rd + kb * 32 * kPitch + 32 * s);
+          kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kDqRowB + (k_rd ^ (s << 5)));
+          vf[buf][kb] = *reinterpret_cast<const bf16x8 *>(vt + kb * 32 * kDqRowB + (k_rd ^ (s << 5)));
+        }
+      };
+#pragma unroll
+      for (int s = 0; s < kPf; ++s) load_kv(s, s);
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int m = 0; m < MSUB; ++m) {
-            sacc[m][kb] = mfma32(kf, qf[m][s], sacc[m][kb]);
-            dpacc[m][kb] = mfma32(vf, dof[m][s], dpacc[m][kb]);
+            sacc[m][kb] = mfma32(kf[s % kPf][kb], qf[m][s], sacc[m][kb]);
+            dpacc[m][kb] = mfma32(vf[s % kPf][kb], dof[m][s], dpacc[m][kb]);
           }
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + kPf < 8) load_kv(s + kPf, s % kPf);
+        if (has_next && s < kLdW) issue_kv(j + 1, stage ^ 1, s);
       }
       // ---- P, dS (one query row per lane) and the bf16 B operand of the dQ product
       const bool need_mask = key0 + kDqKV - 1 > lim_first;
@@ -560,18 +569,29 @@ __global__ __launch_bounds__(256, (MSUB == 1 ? 2 : 1)) void ca_bwd_dq_kernel(Bwd
         }
       }
       // ---- dQ^T += K^T dS^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
+      constexpr int kPfT = 4;
+      bf16x4 ktf[kPfT][2];
+      auto load_t = [&](int u, int buf) {  // u = 4*t + db
+        const uint8_t *kp = kt + 16 * (u >> 2) * kDqRowB;
+        ktf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(kp + (t_rd ^ ((u & 3) << 5))));
+        ktf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(kp + 8 * kDqRowB + (t_rd ^ ((u & 3) << 5) ^ 16)));
+      };
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int u = 0; u < kPfT; ++u) load_t(u, u);
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const uint8_t *kp = kt + t_rd + 16 * t * kPitch + 32 * db;
-          const bf16x8 ktf = cat4(lds_read_tr((const DISTCA_LDS void *)kp), lds_read_tr((const DISTCA_LDS void *)(kp + 8 * kPitch)));
+      for (int u = 0; u < 16; ++u) {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int m = 0; m < MSUB; ++m) dqacc[m][db] = mfma32(ktf, dsf[m][t], dqacc[m][db]);
-        }
+        for (int m = 0; m < MSUB; ++m) dqacc[m][u & 3] = mfma32(cat4(ktf[u % kPfT][0], ktf[u % kPfT][1]), dsf[m][u >> 2], dqacc[m][u & 3]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u + kPfT < 16) load_t(u + kPfT, u % kPfT);
       }
+    } else if (has_next) {
+      // nothing to compute in this tile: still fetch this wave's share of the next one
+#pragma unroll
+      for (int i = 0; i < kLdW; ++i) issue_kv(j + 1, stage ^ 1, i);
     }
-    if (has_next) store_tile(stage ^ 1);
+    wait_vm0();
     __syncthreads();
   }
 
@@ -744,6 +764,7 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
     const int64_t grid = max_items * p->num_heads_kv;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_kv);
+    a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     if (alias)
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
@@ -759,8 +780,9 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
     const int64_t grid = max_items * p->num_heads_kv;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_q);
+    a.zero_row = ws + w.sched_q + sched_zero_row_off(p->num_tasks, max_items);
     ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
-    hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(256), kDqLds, s, a);
+    hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
   }
   if (alias) {
     hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (__bf16 *)dk, kv_elems / 8);

@@ -9,7 +9,10 @@
 namespace distca {
 
 constexpr int kHeadDim = 128;
-constexpr int kWaves = 4;  // waves per workgroup of the dQ kernel
+#ifndef DISTCA_DQ_WAVES
+#define DISTCA_DQ_WAVES 8
+#endif
+constexpr int kWaves = DISTCA_DQ_WAVES;  // waves per workgroup of the dQ kernel
 
 // Forward and dQ kernels: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles
 // of 64 keys.  One sub-tile keeps a wave under 256 registers, so a compute unit holds eight waves.
