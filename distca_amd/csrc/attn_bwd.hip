@@ -151,11 +151,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // Rows past the task (and a group's last block when it does not exist) are clamped to the
   // task's last row so that the loads stay in bounds, and marked by lim = -1 (every key masked).
   auto div_group = [&](int n) { return a.group_magic ? (int)__umulhi((uint32_t)n, a.group_magic) : n; };
-  auto issue_tile = [&](int stage, int mbx) {
+  // The fetch of one block in three pieces: row statistics, rows 0-3, rows 4-7 of this wave's share.
+  // (Issuing them between the MFMAs of phase A, as the forward kernel does, measured 2 % slower here:
+  // the other group is in its LDS-bound phase C at that time.)
+  auto issue_piece = [&](int stage, int mbx, int piece) {
     const int tile = kTileOff + (stage * 2 + grp) * kTileBytes;
     const int stat = kStatOff + (stage * 2 + grp) * kStatBytes;
     const bool blk_ok = mbx >= mb0;
-    {  // row statistics: lanes 0..7 take one row each
+    if (piece == 0) {  // row statistics: lanes 0..7 take one row each
       const int rl = kbw * 8 + (lane & 7);
       const int rho = mbx * kBM + rl;
       const bool ok = blk_ok && rho < nrows;
@@ -170,23 +173,27 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
         lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
         lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
       }
-    }
-    // Q and dO: one instruction fills four rows; lane p brings the chunk that belongs at chunk
-    // position p%16 of row p/16
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    } else {
+      // Q and dO: one instruction fills four rows; lane p brings the chunk that belongs at chunk
+      // position p%16 of row p/16.  Rows that do not exist read the zero row.
+      const int i = piece - 1;
       const int rl = kbw * 8 + 4 * i + (lane >> 4);
       const int rho = mbx * kBM + rl;
       const bool ok = blk_ok && rho < nrows;
-      const int rc = ok ? rho : nrows - 1;
-      const int tok = div_group(rc);
-      const int hg = rc - tok * G;
+      const int tok = div_group(ok ? rho : 0);
+      const int hg = (ok ? rho : 0) - tok * G;
       const int chunk = (lane & 15) ^ tile_swz(rl);
-      const int64_t eo = qbase + (int64_t)(tok * a.hq + hg) * kHeadDim + chunk * 8;
+      const int64_t eo = qbase + (int64_t)(tok * a.hq + hg) * kHeadDim;
+      const __bf16 *qs = ok ? a.q + eo : reinterpret_cast<const __bf16 *>(a.zero_row);
+      const __bf16 *ds = ok ? a.dout + eo : reinterpret_cast<const __bf16 *>(a.zero_row);
       const uint32_t dst = lds0 + tile + (kbw * 8 + 4 * i) * kTileRow;
-      lds_direct_load16_ptr(a.q + eo, dst + kTileQ);
-      lds_direct_load16_ptr(a.dout + eo, dst + kTileDO);
+      lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
+      lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
     }
+  };
+  auto issue_tile = [&](int stage, int mbx) {
+#pragma unroll
+    for (int piece = 0; piece < 3; ++piece) issue_piece(stage, mbx, piece);
   };
 
   const float c = a.scale * kLog2e;
