@@ -20,10 +20,8 @@
 // (16-byte reads), V through the transposing LDS read.
 //
 // K/V tiles go from global memory straight into LDS (LDS-direct loads, four 256-byte rows per
-// instruction, rows unpadded with swizzled 16-byte chunks, see tile_swz).  The eight load
-// instructions a wave contributes to the next tile are issued one at a time between the MFMAs
-// of the current tile's S phase: issued in one burst after the barrier, every wave of the
-// compute unit queues at the vector memory unit at the same moment and the MFMA pipe idles.
+// instruction, rows unpadded with swizzled 16-byte chunks, see tile_swz), one period ahead of
+// their use.
 #include "api_util.h"
 #include "attn_cfg.h"
 #include "common.h"
@@ -34,8 +32,8 @@ namespace {
 constexpr int kRowB = 256;    // bytes per K or V row in LDS (unpadded; chunk c of row r sits at c ^ tile_swz(r))
 constexpr int kKTile = kFwdKV * kRowB;
 constexpr int kVTile = kFwdKV * kRowB;
-constexpr int kStage = kKTile + kVTile;
-constexpr int kFwdLds = 2 * kStage;
+constexpr int kKOff = 0, kVOff = 2 * kKTile;  // two K stages, then two V stages
+constexpr int kFwdLds = 2 * kKTile + 2 * kVTile;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -129,20 +127,21 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int uwave = __builtin_amdgcn_readfirstlane(wave);
   const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
   const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
-  // a wave brings kRowsW rows of the K tile and of the V tile: instructions 0 .. kLdW/2-1 fetch K
-  // rows kRowsW*w + 4i .. +3, the other half the same rows of V
-  constexpr int kRowsW = kFwdKV / kFwdWaves, kLdW = 2 * (kRowsW / 4);
-  auto issue_kv = [&](int j, int stage, int i) {
-    const bool is_k = i < kLdW / 2;
-    const int ii = is_k ? i : i - kLdW / 2;
-    const int r = kRowsW * uwave + 4 * ii + (lane >> 4);
-    const int key = j * kFwdKV + r;
-    const int chunk = (lane & 15) ^ tile_swz(r);
-    const __bf16 *src = (is_k ? kbase : vbase) + (int64_t)key * kv_stride;
-    if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
-    const uint32_t dst = lds0 + stage * kStage + (is_k ? 0 : kKTile) + (kRowsW * uwave + 4 * ii) * kRowB;
-    lds_direct_load16_ptr(src + chunk * 8, dst);
+  // a wave brings kRowsW rows of a K tile or of a V tile, four rows per instruction
+  constexpr int kRowsW = kFwdKV / kFwdWaves, kLdW = kRowsW / 4;
+  auto issue_rows = [&](const __bf16 *base, int j, uint32_t tile_off) {
+#pragma unroll
+    for (int i = 0; i < kLdW; ++i) {
+      const int r = kRowsW * uwave + 4 * i + (lane >> 4);
+      const int key = j * kFwdKV + r;
+      const int chunk = (lane & 15) ^ tile_swz(r);
+      const __bf16 *src = base + (int64_t)key * kv_stride;
+      if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
+      lds_direct_load16_ptr(src + chunk * 8, lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
+    }
   };
+  auto issue_k = [&](int j) { issue_rows(kbase, j, kKOff + (j & 1) * kKTile); };
+  auto issue_v = [&](int j) { issue_rows(vbase, j, kVOff + (j & 1) * kVTile); };
 
   // ---- accumulators
   f32x16 oacc[MSUB][4];
@@ -165,131 +164,148 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
   const int v_rd = (4 * g + i4) * kRowB + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*db ^ 16*hi
 
-  if (ntiles > 0) {
+  f32x16 sacc[MSUB][2];
+  bf16x8 pf[MSUB][4];
+  auto tile_active = [&](int j) { return wave_live && j * kFwdKV <= lim_last; };
+
+  // ---- S^T = K Q^T : [64 keys] x [32*MSUB rows]
+  auto phase_s = [&](int j) {
+    const uint8_t *kt = lds + kKOff + (j & 1) * kKTile;
 #pragma unroll
-    for (int i = 0; i < kLdW; ++i) issue_kv(0, 0, i);
-  }
-  wait_vm0();
-  __syncthreads();
-
-  for (int j = 0; j < ntiles; ++j) {
-    const int stage = j & 1;
-    const uint8_t *kt = lds + stage * kStage;
-    const uint8_t *vt = kt + kKTile;
-    const bool has_next = j + 1 < ntiles;
-
+    for (int m = 0; m < MSUB; ++m)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[m][kb][r] = 0.f;
+    constexpr int kPf = 2;  // K fragments are requested kPf steps before the MFMAs that use them
+    bf16x8 kf[kPf][2];
+    auto load_k = [&](int s, int buf) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kRowB + (k_rd ^ (s << 5)));
+    };
+#pragma unroll
+    for (int s = 0; s < kPf; ++s) load_k(s, s);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int m = 0; m < MSUB; ++m) sacc[m][kb] = mfma32(kf[s % kPf][kb], qf[m][s], sacc[m][kb]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + kPf < 8) load_k(s + kPf, s % kPf);
+    }
+  };
+  // ---- mask, online softmax (log2 domain, one query row per lane pair), P as bf16 B operand
+  auto phase_x = [&](int j) {
     const int key0 = j * kFwdKV;
-    const bool active = wave_live && key0 <= lim_last;
-    bf16x8 pf[MSUB][4];
-    if (active) {
-      // ---- S^T = K Q^T : [64 keys] x [32*MSUB rows]
-      f32x16 sacc[MSUB][2];
+    if (key0 + kFwdKV - 1 > lim_first) {  // the tile straddles the diagonal or the end of the prefix
 #pragma unroll
       for (int m = 0; m < MSUB; ++m)
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sacc[m][kb][r] = 0.f;
-      // K fragments are requested kPf steps before the MFMAs that use them
-      constexpr int kPf = 2;
-      bf16x8 kf[kPf][2];
-      auto load_k = [&](int s, int buf) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kRowB + (k_rd ^ (s << 5)));
-      };
-#pragma unroll
-      for (int s = 0; s < kPf; ++s) load_k(s, s);
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int m = 0; m < MSUB; ++m) sacc[m][kb] = mfma32(kf[s % kPf][kb], qf[m][s], sacc[m][kb]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (s + kPf < 8) load_k(s + kPf, s % kPf);
-        if (has_next && s < kLdW) issue_kv(j + 1, stage ^ 1, s);  // next tile, one instruction per step
-      }
-      // ---- mask the tiles that straddle the diagonal or the end of the prefix
-      if (key0 + kFwdKV - 1 > lim_first) {
-#pragma unroll
-        for (int m = 0; m < MSUB; ++m)
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = key0 + kb * 32 + acc_row(r, g);
-              if (key > lim[m]) sacc[m][kb][r] = -INFINITY;
-            }
-      }
-      // ---- online softmax (log2 domain), one query row per lane pair
-#pragma unroll
-      for (int m = 0; m < MSUB; ++m) {
-        float mx = sacc[m][0][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, sacc[m][kb][r]);
-        mx = pair_max(mx);
-        const float m_new = __builtin_fmaxf(m_run[m], mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        if (__any(m_new != m_run[m])) {
-          const float alpha = fast_exp2((m_run[m] - m_use) * c);
-          l_run[m] *= alpha;
-#pragma unroll
-          for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[m][db][r] *= alpha;
-          m_run[m] = m_new;
-        }
-        const float mc = -m_use * c;
-        float sum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, mc));
-            sacc[m][kb][r] = p;
-            sum += p;
+            const int key = key0 + kb * 32 + acc_row(r, g);
+            if (key > lim[m]) sacc[m][kb][r] = -INFINITY;
           }
-        l_run[m] += sum;
+    }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int kb = t >> 1, r0 = 8 * (t & 1);
-          pf[m][t] = cvt8(sacc[m][kb][r0], sacc[m][kb][r0 + 1], sacc[m][kb][r0 + 2], sacc[m][kb][r0 + 3], sacc[m][kb][r0 + 4],
-                          sacc[m][kb][r0 + 5], sacc[m][kb][r0 + 6], sacc[m][kb][r0 + 7]);
+    for (int m = 0; m < MSUB; ++m) {
+      float mx = sacc[m][0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, sacc[m][kb][r]);
+      mx = pair_max(mx);
+      const float m_new = __builtin_fmaxf(m_run[m], mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      if (__any(m_new != m_run[m])) {
+        const float alpha = fast_exp2((m_run[m] - m_use) * c);
+        l_run[m] *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[m][db][r] *= alpha;
+        m_run[m] = m_new;
+      }
+      const float mc = -m_use * c;
+      float sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, mc));
+          sacc[m][kb][r] = p;
+          sum += p;
         }
+      l_run[m] += sum;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int kb = t >> 1, r0 = 8 * (t & 1);
+        pf[m][t] = cvt8(sacc[m][kb][r0], sacc[m][kb][r0 + 1], sacc[m][kb][r0 + 2], sacc[m][kb][r0 + 3], sacc[m][kb][r0 + 4],
+                        sacc[m][kb][r0 + 5], sacc[m][kb][r0 + 6], sacc[m][kb][r0 + 7]);
       }
     }
-    // a wave with nothing to compute in this tile still fetches its share of the next one (the
-    // other LDS stage: its last readers finished before the barrier that ended the previous iteration)
-    if (!active && has_next) {
+  };
+  // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
+  auto phase_pv = [&](int j) {
+    const uint8_t *vt = lds + kVOff + (j & 1) * kVTile;
+    constexpr int kPfV = 4;  // V^T fragments are requested four MFMAs ahead
+    bf16x4 vf[kPfV][2];
+    auto load_v = [&](int u, int buf) {  // u = 4*t + db
+      const uint8_t *vp = vt + 16 * (u >> 2) * kRowB;
+      vf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(vp + (v_rd ^ ((u & 3) << 5))));
+      vf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kRowB + (v_rd ^ ((u & 3) << 5) ^ 16)));
+    };
 #pragma unroll
-      for (int i = 0; i < kLdW; ++i) issue_kv(j + 1, stage ^ 1, i);
+    for (int u = 0; u < kPfV; ++u) load_v(u, u);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < MSUB; ++m) oacc[m][u & 3] = mfma32(cat4(vf[u % kPfV][0], vf[u % kPfV][1]), pf[m][u >> 2], oacc[m][u & 3]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (u + kPfV < 16) load_v(u + kPfV, u % kPfV);
     }
+  };
 
-    if (active) {
-      // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
-      constexpr int kPfV = 4;  // V^T fragments are requested four MFMAs ahead
-      bf16x4 vf[kPfV][2];
-      auto load_v = [&](int u, int buf) {  // u = 4*t + db
-        const uint8_t *vp = vt + 16 * (u >> 2) * kRowB;
-        vf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(vp + (v_rd ^ ((u & 3) << 5))));
-        vf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kRowB + (v_rd ^ ((u & 3) << 5) ^ 16)));
-      };
-#pragma unroll
-      for (int u = 0; u < kPfV; ++u) load_v(u, u);
-#pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int m = 0; m < MSUB; ++m) oacc[m][u & 3] = mfma32(cat4(vf[u % kPfV][0], vf[u % kPfV][1]), pf[m][u >> 2], oacc[m][u & 3]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (u + kPfV < 16) load_v(u + kPfV, u % kPfV);
-      }
+  // The waves form two groups (0-3, 4-7; a SIMD holds one wave of each) that run half a period
+  // apart, so that one group's MFMA phases coincide with the other's softmax arithmetic instead
+  // of both queueing for the same pipe.  Between consecutive workgroup barriers b0, b1, b2, ...
+  //   [b(2p),   b(2p+1)):  group 0: PV(p-1), S(p)     group 1: softmax(p-1)
+  //   [b(2p+1), b(2p+2)):  group 0: softmax(p)        group 1: PV(p-1), S(p)
+  // Tile p of K is read between b(2p) and b(2p+2), tile p of V between b(2p+2) and b(2p+4); every
+  // wave requests K(p+1) and V(p) right after b(2p), into the stages whose last readers finished
+  // before that barrier, and waits for its own requests before b(2p+2).
+  const int grp = uwave >> 2;
+  if (ntiles > 0) issue_k(0);
+  wait_vm0();
+  __syncthreads();  // b0
+  if (grp == 0) {
+    for (int p = 0; p <= ntiles; ++p) {
+      if (p + 1 < ntiles) issue_k(p + 1);
+      if (p < ntiles) issue_v(p);
+      if (p > 0 && tile_active(p - 1)) phase_pv(p - 1);
+      const bool act = p < ntiles && tile_active(p);
+      if (act) phase_s(p);
+      __syncthreads();
+      if (act) phase_x(p);
+      wait_vm0();
+      __syncthreads();
     }
-    wait_vm0();
-    __syncthreads();
+  } else {
+    for (int p = 0; p <= ntiles; ++p) {
+      if (p + 1 < ntiles) issue_k(p + 1);
+      if (p < ntiles) issue_v(p);
+      const bool act_prev = p > 0 && tile_active(p - 1);
+      if (act_prev) phase_x(p - 1);
+      __syncthreads();
+      if (act_prev) phase_pv(p - 1);
+      if (p < ntiles && tile_active(p)) phase_s(p);
+      wait_vm0();
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: normalise, write O (bf16) and LSE (fp32, natural log)
