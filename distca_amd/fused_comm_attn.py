@@ -17,7 +17,8 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .dispatch import (post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_with_lse, pre_a2a_qkv)
+from .dispatch import (post_a2a_attn_out, post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_grad_resend_qkv,
+                       pre_a2a_attn_out_with_lse, pre_a2a_qkv)
 
 
 @dataclass
@@ -310,3 +311,66 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
         is_fwd=False, kv_grad_copy_shard_mask=meta.main_copy_mask,
         pre_a2a_grad_acc_args=(meta.num_copies, meta.copy_start_id, meta.k_grad_send_seq_tokens), buffer=send_buffer)
     return dq, dk, dv
+
+
+# ---------------------------------------------------------------------------------------
+# The same tick driven by AlltoAllMetadata, and the linear side of it (what the reference's
+# autograd functions do around the all-to-all): fused_comm_attn.py:287-461 and :464-526.
+# ---------------------------------------------------------------------------------------
+def fused_comm_attn_forward(recv_buffer: Tensor, send_buffer: Tensor, packed_seq_params, fa_args: FlashAttnArgs,
+                            dtype: torch.dtype = torch.bfloat16):
+    """FusedCommAttn.forward on explicit buffers: `recv_buffer` holds what the q/k/v all-to-all
+    delivered (qkv_fwd_metadata.recv_memcpy_metadata), `send_buffer` receives the [out | lse] reply
+    (attn_out_fwd_metadata.send_memcpy_metadata).  Returns (attn_out, softmax_lse [Hq, T])."""
+    qkv, out = packed_seq_params.qkv_fwd_metadata, packed_seq_params.attn_out_fwd_metadata
+    q_off, k_off, v_off = qkv.recv_memcpy_metadata
+    meta = ServerFwdMeta(qkv.seq_lens[0].recv_seqlens, qkv.seq_lens[1].recv_seqlens, q_off, k_off, v_off,
+                         out.seq_lens[0].send_seqlens, out.send_memcpy_metadata[0],
+                         tuple(qkv.tensor_shape[0].recv_shape), tuple(qkv.tensor_shape[1].recv_shape))
+    return ca_server_forward(recv_buffer, send_buffer, meta, packed_seq_params, fa_args, dtype)
+
+
+def fused_comm_attn_backward(recv_buffer: Tensor, send_buffer: Tensor, packed_seq_params, fa_args: FlashAttnArgs,
+                             dtype: torch.dtype = torch.bfloat16):
+    """FusedCommAttn.backward / dummy_backward_single_sided (fused_comm_attn.py:407-461, 529-642)
+    on explicit buffers: request per attn_out_bwd_metadata, gradient reply per qkv_bwd_metadata."""
+    req, grad = packed_seq_params.attn_out_bwd_metadata, packed_seq_params.qkv_bwd_metadata
+    bwd = packed_seq_params.bwd_packed_seq_params
+    q_off, k_off, v_off = req.recv_memcpy_metadata
+    gq_off, gk_off, gv_off = grad.send_memcpy_metadata
+    tq = int(req.tensor_shape[0].recv_shape[0])
+    hq_d = fa_args.num_heads_q * fa_args.head_dim
+    d = grad.kv_grad_send_dedup
+    meta = ServerBwdMeta(req.seq_lens[0].recv_seqlens, req.seq_lens[1].recv_seqlens, q_off, k_off, v_off,
+                         grad.seq_lens[0].send_seqlens, grad.seq_lens[1].send_seqlens, gq_off, gk_off, gv_off,
+                         d.main_copy_mask, d.num_copies, d.copy_start_id, (tq, hq_d), (tq, fa_args.num_heads_q),
+                         tuple(req.tensor_shape[1].recv_shape))
+    return ca_server_backward(recv_buffer, send_buffer, meta, fa_args, bwd.cu_seqlens_q, bwd.cu_seqlens_kv,
+                              bwd.max_seqlen_q, bwd.max_seqlen_kv, dtype)
+
+
+def post_a2a_attn_out_with_lse(recv_buffer: Tensor, q: Tensor, num_heads_q: int, metadata, dtype: torch.dtype = None):
+    """Linear side, forward of the reference's autograd function of the same name
+    (fused_comm_attn.py:468-506): unpack the [out | lse | pad] tokens of the reply and split them.
+    Returns (attn_out [T, 1, Hq*D] in q's dtype, softmax_lse_bytes [T, Hq*4] uint8)."""
+    dtype = dtype or q.dtype
+    recv_shape = tuple(metadata.tensor_shape[0].recv_shape)
+    recv = torch.empty(recv_shape, dtype=torch.uint8, device=recv_buffer.device)
+    post_a2a_attn_out(recv, metadata.seq_lens[0].recv_seqlens, *metadata.recv_memcpy_metadata, buffer=recv_buffer)
+    itemsize = torch.empty((), dtype=dtype).element_size()
+    hidden_bytes = int(q.numel() // q.shape[0]) * itemsize
+    lse_bytes = num_heads_q * 4
+    attn_out = recv[:, :hidden_bytes].contiguous().view(dtype).unsqueeze(1)
+    softmax_lse_bytes = recv[:, hidden_bytes:hidden_bytes + lse_bytes]
+    return attn_out, softmax_lse_bytes
+
+
+def post_a2a_attn_out_with_lse_backward(send_buffer: Tensor, grad_attn_out: Tensor, attn_out: Tensor, softmax_lse_bytes: Tensor,
+                                        q: Tensor, k: Tensor, v: Tensor, bwd_attn_out_qkv_metadata):
+    """Linear side, backward of the same function (fused_comm_attn.py:508-526): pack the request
+    [dO | O | lse | q | pad] and the K/V shards for the attention server."""
+    flat = lambda t: t.reshape(t.shape[0], -1)
+    md = bwd_attn_out_qkv_metadata
+    pre_a2a_attn_out_grad_resend_qkv(
+        flat(grad_attn_out), flat(attn_out), softmax_lse_bytes, flat(q), flat(k), flat(v), md.kv_replica_mask,
+        md.seq_lens[0].send_seqlens, md.seq_lens[1].send_seqlens, *md.send_memcpy_metadata, buffer=send_buffer)

@@ -71,6 +71,63 @@ class DedupGradSumMetadata:
                                     _dev(self.main_copy_mask, torch.int8, device))
 
 
+def _slice_or_none(x, rank):
+    return None if x is None else x[rank]
+
+
+@dataclass
+class AlltoAllMetadata:
+    """Everything one all-to-all of the CA path needs (fields and meaning of
+    distca/runtime/metadata.py:70-100): the transport's per-peer displacements and sizes
+    (`fa2a_metadata`: sender_send_offset, sender_transfer_sz, sender_recv_offset,
+    recver_transfer_sz, in bytes), the byte offset of every shard in the send buffer
+    (`send_memcpy_metadata`, ordered by the sender's shards; for K/V as [cp, shard]) and in the
+    receive buffer (`recv_memcpy_metadata`, ordered by the receiver's shards), the shard lengths
+    and tensor shapes on either side, the K/V replica mask of the sender and, for the gradient
+    direction, the duplicate-gradient metadata."""
+    fa2a_metadata: Tuple[Tensor, Tensor, Tensor, Tensor]
+    send_memcpy_metadata: Sequence[_TensorOrList]
+    recv_memcpy_metadata: Sequence[_TensorOrList]
+    my_rank_send_offset: Union[int, List[int]]
+    my_rank_recv_offset: Union[int, List[int]]
+    my_rank_send_sz: Union[int, List[int]]
+    seq_lens: Sequence[SeqLens]
+    tensor_shape: Sequence[LogicalShape]
+    kv_replica_mask: Optional[_TensorOrList] = None
+    kv_grad_send_dedup: Optional[Union[DedupGradSumMetadata, Sequence[DedupGradSumMetadata]]] = None
+    single_stream: bool = False
+    send_num_seqs: Optional[Sequence[int]] = None
+    recv_num_seqs: Optional[Sequence[int]] = None
+    max_cp_degree: Optional[int] = None
+
+    def get_slice(self, rank):
+        """The metadata of one rank out of the stacked per-rank form (metadata.py:177-198)."""
+        return AlltoAllMetadata(
+            tuple(t[rank] for t in self.fa2a_metadata),
+            tuple(t[rank] for t in self.send_memcpy_metadata),
+            tuple(t[rank] for t in self.recv_memcpy_metadata),
+            self.my_rank_send_offset[rank], self.my_rank_recv_offset[rank], self.my_rank_send_sz[rank],
+            tuple(sl.get_slice(rank) for sl in self.seq_lens),
+            tuple(ts.get_slice(rank) for ts in self.tensor_shape),
+            kv_replica_mask=_slice_or_none(self.kv_replica_mask, rank),
+            kv_grad_send_dedup=_slice_or_none(self.kv_grad_send_dedup, rank),
+            single_stream=self.single_stream)
+
+    def normalize(self, device="cuda"):
+        """To device with the dtypes the kernels read (metadata.py:200-220): transport
+        displacements uint64, shard offsets int64, masks int8."""
+        return AlltoAllMetadata(
+            tuple(_dev(t, torch.uint64, device) for t in self.fa2a_metadata),
+            tuple(_dev(t, torch.int64, device) for t in self.send_memcpy_metadata),
+            tuple(_dev(t, torch.int64, device) for t in self.recv_memcpy_metadata),
+            self.my_rank_send_offset, self.my_rank_recv_offset, self.my_rank_send_sz,
+            tuple(t.normalize(device) for t in self.seq_lens), self.tensor_shape,
+            kv_replica_mask=_dev(self.kv_replica_mask, torch.int8, device) if self.kv_replica_mask is not None else None,
+            kv_grad_send_dedup=self.kv_grad_send_dedup.normalize(device) if self.kv_grad_send_dedup is not None else None,
+            single_stream=self.single_stream, send_num_seqs=self.send_num_seqs, recv_num_seqs=self.recv_num_seqs,
+            max_cp_degree=self.max_cp_degree)
+
+
 def get_attn_metadata(seqlens_q, seqlens_kv=None, get_packed_seq_params: bool = False):
     """cu_seqlens / max_seqlen of a task list (one tensor) or of one list per rank."""
     from .fused_comm_attn import PackedSeqParams
@@ -232,3 +289,84 @@ def server_metas(plan: SingleRankPlan, device="cuda"):
                         i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(gq), i64(gk), i64(gv),
                         d.main_copy_mask, d.num_copies, d.copy_start_id, (tq, hq_d), (tq, plan.num_heads_q), (tk, hkv_d))
     return attn, fwd, bwd, (f_recv, f_send, b_recv, b_send)
+
+
+@dataclass
+class PingPangSingleStepPackedSeqParams:
+    """What one layer step carries into the CA path (runtime/megatron/packed_seq_params.py:26-57):
+    the attention-layout cu_seqlens plus the four all-to-all descriptions (q/k/v out and gradients
+    back, attention output out and its gradient back) and the backward's own cu_seqlens."""
+    qkv_format: str = "thd"
+    cu_seqlens_q: Tensor = None
+    cu_seqlens_kv: Tensor = None
+    max_seqlen_q: int = None
+    max_seqlen_kv: int = None
+    qkv_fwd_metadata: AlltoAllMetadata = None
+    qkv_bwd_metadata: AlltoAllMetadata = None
+    attn_out_fwd_metadata: AlltoAllMetadata = None
+    attn_out_bwd_metadata: AlltoAllMetadata = None
+    bwd_packed_seq_params: object = None
+    stream: object = None
+    dispatcher_id: int = None
+    kv_task_offsets: Optional[Tensor] = None
+
+    def to_device(self, device="cuda"):
+        to_i32 = lambda t: None if t is None else _dev(t, torch.int32, device)
+        to_int = lambda x: None if x is None else int(x)
+        bwd = self.bwd_packed_seq_params
+        if bwd is not None:
+            bwd = type(bwd)(cu_seqlens_q=to_i32(bwd.cu_seqlens_q), cu_seqlens_kv=to_i32(bwd.cu_seqlens_kv),
+                            max_seqlen_q=to_int(bwd.max_seqlen_q), max_seqlen_kv=to_int(bwd.max_seqlen_kv))
+        return PingPangSingleStepPackedSeqParams(
+            self.qkv_format, to_i32(self.cu_seqlens_q), to_i32(self.cu_seqlens_kv), to_int(self.max_seqlen_q),
+            to_int(self.max_seqlen_kv), self.qkv_fwd_metadata.normalize(device), self.qkv_bwd_metadata.normalize(device),
+            self.attn_out_fwd_metadata.normalize(device), self.attn_out_bwd_metadata.normalize(device), bwd, self.stream,
+            self.dispatcher_id, to_i32(self.kv_task_offsets))
+
+
+def single_rank_step_params(plan: SingleRankPlan) -> PingPangSingleStepPackedSeqParams:
+    """The four AlltoAllMetadata of one layer step when the linear rank and the attention rank are
+    the same GPU (world size 1: the transport moves `my_rank_send_sz` bytes from the send buffer's
+    offset 0 to the receive buffer's offset 0).  Host tensors; call to_device() before use."""
+    from .fused_comm_attn import PackedSeqParams
+    t64 = lambda x: torch.tensor([[x]], dtype=torch.int64)
+    tq, tkv = plan.num_q_tokens, plan.num_kv_tokens
+    stored = plan.stored_shard_tokens
+    hq_d, hkv_d = plan.num_heads_q * plan.head_dim, plan.num_heads_kv * plan.head_dim
+    first = torch.tensor([plan.kv_entry_shard.tolist().index(s) for s in range(len(stored))], dtype=torch.int64)
+
+    def qkv_md(backward_request: bool):
+        q_off, k_off, v_off, total = plan.request_layout(backward_request)
+        qb = plan.merged_q_bytes if backward_request else plan.q_bytes * 1
+        send = (q_off, k_off[first].unsqueeze(0), v_off[first].unsqueeze(0))      # K/V as [cp = 1, shard]
+        recv = (q_off, k_off, v_off)
+        seq = (SeqLens(plan.q_seqlens, plan.q_seqlens), SeqLens(stored, plan.kv_entry_tokens))
+        q_cols = qb // plan.itemsize if not backward_request else qb
+        shape = (LogicalShape(torch.Size((tq, q_cols)), torch.Size((tq, q_cols))),
+                 LogicalShape(torch.Size((1, int(stored.sum()), hkv_d)), torch.Size((tkv, hkv_d))))
+        return AlltoAllMetadata((t64(0), t64(total), t64(0), t64(total)), send, recv, 0, 0, total, seq, shape,
+                                kv_replica_mask=torch.ones((len(stored), 1), dtype=torch.int8))
+
+    def grad_md():
+        q_off, k_off, v_off, total = plan.reply_layout(True)
+        send = (q_off, k_off, v_off)                                               # ordered by the server's entries
+        recv = (q_off, k_off[first].unsqueeze(0), v_off[first].unsqueeze(0))
+        seq = (SeqLens(plan.q_seqlens, plan.q_seqlens), SeqLens(plan.kv_entry_tokens, stored))
+        shape = (LogicalShape(torch.Size((tq, hq_d)), torch.Size((tq, hq_d))),
+                 LogicalShape(torch.Size((tkv, hkv_d)), torch.Size((1, int(stored.sum()), hkv_d))))
+        return AlltoAllMetadata((t64(0), t64(total), t64(0), t64(total)), send, recv, 0, 0, total, seq, shape,
+                                kv_replica_mask=torch.ones((len(stored), 1), dtype=torch.int8), kv_grad_send_dedup=plan.dedup)
+
+    def out_md():
+        off, _, _, total = plan.reply_layout(False)
+        seq = (SeqLens(plan.q_seqlens, plan.q_seqlens),)
+        shape = (LogicalShape(torch.Size((tq, plan.out_lse_bytes)), torch.Size((tq, plan.out_lse_bytes))),)
+        return AlltoAllMetadata((t64(0), t64(total), t64(0), t64(total)), (off,), (off,), 0, 0, total, seq, shape)
+
+    attn = get_attn_metadata(plan.q_seqlens, plan.kv_seqlens)
+    bwd = PackedSeqParams(cu_seqlens_q=attn["cu_seqlens_q"], cu_seqlens_kv=attn["cu_seqlens_kv"],
+                          max_seqlen_q=attn["max_seqlen_q"], max_seqlen_kv=attn["max_seqlen_kv"])
+    return PingPangSingleStepPackedSeqParams(
+        "thd", attn["cu_seqlens_q"], attn["cu_seqlens_kv"], attn["max_seqlen_q"], attn["max_seqlen_kv"],
+        qkv_fwd_metadata=qkv_md(False), qkv_bwd_metadata=grad_md(), attn_out_fwd_metadata=out_md(),
+        attn_out_bwd_metadata=qkv_md(True), bwd_packed_seq_params=bwd)

@@ -241,3 +241,60 @@ def test_server_tick_from_single_rank_plan(cuda):
     # a stored shard's gradient is the bf16 sum of up to four per-task bf16 gradients: 4e-2 / 3e-3
     assert_close_bf16(tb(dk, 2), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
     assert_close_bf16(tb(dv, 2), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
+
+
+def test_layer_step_with_alltoall_metadata(cuda):
+    """Linear side and attention server of one layer step on one GPU (world size 1: the all-to-all
+    moves nothing, send and receive buffer are the same memory), every hop through the ops of this
+    package with the reference's metadata objects: pre_a2a_qkv -> FusedCommAttn forward ->
+    post_a2a_attn_out_with_lse; its backward -> FusedCommAttn backward -> post_a2a_qkv(is_fwd=False)."""
+    from distca_amd import metadata
+    from distca_amd.dispatch import post_a2a_qkv, pre_a2a_qkv
+    from distca_amd.fused_comm_attn import (FlashAttnArgs, fused_comm_attn_backward, fused_comm_attn_forward,
+                                            post_a2a_attn_out_with_lse, post_a2a_attn_out_with_lse_backward)
+    docs = [[100, 156, 300], [77]]
+    hq, hkv, d = 8, 2, 128
+    plan = metadata.single_rank_plan(docs, hq, hkv)
+    step = metadata.single_rank_step_params(plan).to_device(cuda)
+    fa_args = FlashAttnArgs(hq, hkv, d)
+    T = plan.num_q_tokens
+    q, k, v, do = make_qkv(T, T, hq, hkv, d, 44)
+    qd, kd, vd, dod = (x.reshape(x.shape[0], -1).to(cuda) for x in (q, k, v, do))
+    new_buf = lambda md: torch.zeros(int(md.my_rank_send_sz), dtype=torch.uint8, device=cuda)
+
+    # forward: linear packs q, k, v (K/V once per stored shard), server answers [out | lse]
+    fwd = step.qkv_fwd_metadata
+    buf = new_buf(fwd)
+    pre_a2a_qkv(qd, kd, vd, fwd.kv_replica_mask, fwd.seq_lens[0].send_seqlens, fwd.seq_lens[1].send_seqlens,
+                *fwd.send_memcpy_metadata, is_fwd=True, buffer=buf)
+    out_buf = new_buf(step.attn_out_fwd_metadata)
+    print("metadata forward", flush=True)
+    fused_comm_attn_forward(buf, out_buf, step, fa_args)
+    attn_out, lse_bytes = post_a2a_attn_out_with_lse(out_buf, qd, hq, step.attn_out_fwd_metadata)
+    torch.cuda.synchronize()
+    cu_doc = np.concatenate([[0], np.cumsum([sum(x) for x in docs])]).astype(np.int32)
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_doc, cu_doc)
+    assert_close_bf16(attn_out.reshape(T, hq, d), ref_out, "out")
+    lse = lse_bytes.contiguous().view(torch.float32)                      # [T, Hq]
+    assert (lse.T.cpu() - ref_lse).abs().max().item() <= 2e-3
+
+    # backward: linear packs [dO | O | lse | q] and K/V again, server returns dq and the summed dk, dv
+    req = step.attn_out_bwd_metadata
+    req_buf = new_buf(req)
+    post_a2a_attn_out_with_lse_backward(req_buf, dod, attn_out, lse_bytes.contiguous(), qd, kd, vd, req)
+    grad = step.qkv_bwd_metadata
+    grad_buf = new_buf(grad)
+    print("metadata backward", flush=True)
+    fused_comm_attn_backward(req_buf, grad_buf, step, fa_args)
+    dq = torch.zeros_like(qd)
+    dk_planes = torch.zeros((1,) + tuple(kd.shape), dtype=kd.dtype, device=cuda)
+    dv_planes = torch.zeros_like(dk_planes)
+    post_a2a_qkv(dq, dk_planes, dv_planes, grad.kv_replica_mask, grad.seq_lens[0].recv_seqlens, grad.seq_lens[1].recv_seqlens,
+                 *grad.recv_memcpy_metadata, is_fwd=False, buffer=grad_buf)
+    torch.cuda.synchronize()
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=attn_out.cpu().reshape(T, hq, d),
+                                              softmax_lse=lse.T.contiguous().cpu())
+    assert_close_bf16(dq.reshape(T, hq, d), ref_dq, "dq")
+    # up to three per-task bf16 gradients summed in bf16 per stored shard: 4e-2 / 3e-3
+    assert_close_bf16(dk_planes.sum(0).reshape(T, hkv, d), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
+    assert_close_bf16(dv_planes.sum(0).reshape(T, hkv, d), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)

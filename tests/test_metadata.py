@@ -81,3 +81,39 @@ def test_plan_drives_the_oracle_round_trip():
     summed = g.clone()
     fa2a.grad_sum(summed, p.dedup.num_copies.numpy(), p.dedup.copy_start_id.numpy(), p.kv_entry_tokens.numpy())
     assert torch.equal(summed[0:3], g[0:3] + g[3:6])              # k0's copy in task 1 folded into the main copy
+
+
+def test_single_rank_step_params_are_consistent():
+    """The four AlltoAllMetadata of a step agree with each other: what one side sends is what the
+    other receives, sizes tile the buffers, normalize() yields the dtypes the kernels read."""
+    p = metadata.single_rank_plan([[4, 2, 3], [6]], 6, 2)
+    step = metadata.single_rank_step_params(p)
+    for md in (step.qkv_fwd_metadata, step.qkv_bwd_metadata, step.attn_out_fwd_metadata, step.attn_out_bwd_metadata):
+        assert md.fa2a_metadata[1].item() == md.my_rank_send_sz == md.fa2a_metadata[3].item()
+        n = md.normalize("cpu")
+        assert all(t.dtype == torch.uint64 for t in n.fa2a_metadata)
+        assert all(t.dtype == torch.int64 for t in n.send_memcpy_metadata + n.recv_memcpy_metadata)
+    fwd, grad = step.qkv_fwd_metadata, step.qkv_bwd_metadata
+    assert fwd.seq_lens[1].send_seqlens.tolist() == [4, 2, 3, 6]                  # stored shards
+    assert fwd.seq_lens[1].recv_seqlens.tolist() == [4, 4, 2, 4, 2, 3, 6]        # prefix entries per task
+    assert fwd.send_memcpy_metadata[1].shape == (1, 4) and fwd.kv_replica_mask.shape == (4, 1)
+    # every entry of a stored shard unpacks from the bytes its single copy was packed to
+    sent = fwd.send_memcpy_metadata[1][0]
+    for e, s_ in enumerate(p.kv_entry_shard.tolist()):
+        assert fwd.recv_memcpy_metadata[1][e] == sent[s_]
+    # gradients: the server sends entries (masked to main copies), the linear side receives stored shards
+    assert grad.seq_lens[1].send_seqlens.tolist() == fwd.seq_lens[1].recv_seqlens.tolist()
+    assert grad.kv_grad_send_dedup.main_copy_mask.tolist() == [1, 0, 1, 0, 0, 1, 1]
+    dev = step.to_device("cpu")
+    assert dev.cu_seqlens_q.dtype == torch.int32 and dev.bwd_packed_seq_params.cu_seqlens_kv.dtype == torch.int32
+
+
+def test_alltoall_metadata_get_slice():
+    two = metadata.AlltoAllMetadata(
+        tuple(torch.arange(4).reshape(2, 2) + i for i in range(4)), (torch.arange(6).reshape(2, 3),), (torch.arange(6).reshape(2, 3) * 2,),
+        [0, 10], [0, 20], [5, 6], (metadata.SeqLens(torch.ones(2, 3), torch.ones(2, 3) * 2),),
+        (metadata.LogicalShape([torch.Size((3, 8)), torch.Size((4, 8))], [torch.Size((5, 8)), torch.Size((6, 8))]),))
+    r1 = two.get_slice(1)
+    assert r1.my_rank_send_offset == 10 and r1.my_rank_send_sz == 6
+    assert r1.send_memcpy_metadata[0].tolist() == [3, 4, 5] and r1.recv_memcpy_metadata[0].tolist() == [6, 8, 10]
+    assert r1.seq_lens[0].recv_seqlens.tolist() == [2, 2, 2] and r1.tensor_shape[0].recv_shape == torch.Size((6, 8))
