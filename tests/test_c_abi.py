@@ -115,3 +115,53 @@ def test_schedule_host_reports_needed_capacity():
     # a short array receives the first max_items items; the full count is still returned
     assert lib.distca_ca_schedule_host(0, cu.ctypes.data, cu.ctypes.data, ctypes.byref(p), small.ctypes.data, 1) == n
     assert small[0, 0] == 0 and (small[1] == -7).all()
+
+
+def test_attention_argument_errors_are_reported_before_any_launch():
+    """Null, misaligned and undersized arguments come back as error codes with a message; the
+    pointers are fake host addresses, so reaching a kernel launch would fail differently."""
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    base = (ctypes.addressof(buf) + 255) // 256 * 256
+    ptr = ctypes.c_void_p(base)
+    odd = ctypes.c_void_p(base + 2)
+    p = _p()
+    need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
+    args = lambda **kw: [kw.get("q", ptr), ptr, ptr, ptr, ptr, ptr, ptr, None, ctypes.byref(p), kw.get("ws", ptr), kw.get("ws_bytes", need), None]
+    assert lib.distca_ca_fwd(*args(ws_bytes=need - 1)) == -3
+    assert b"workspace" in lib.distca_last_error()
+    assert lib.distca_ca_fwd(*args(ws=None)) == -3
+    assert lib.distca_ca_fwd(*args(q=odd)) == -1
+    assert b"aligned" in lib.distca_last_error()
+    assert lib.distca_ca_fwd(*args(q=None)) == -1
+    # backward: deterministic together with shared KV rows is refused, as documented
+    pd = _p(deterministic=1)
+    needb = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(pd))
+    bargs = [ptr] * 9 + [ptr, ptr, ptr, ctypes.byref(pd), ptr, needb, None]
+    assert lib.distca_ca_bwd(*bargs) == -2
+    assert b"deterministic" in lib.distca_last_error()
+    bargs[11] = None                                          # no kv_task_offsets: passes validation up to the workspace check
+    bargs[14] = 64                                             # (the size query covers the shared-KV form; 64 B is too small for either)
+    assert lib.distca_ca_bwd(*bargs) == -3
+    # a batch without tasks or rows is a no-op that touches nothing
+    assert lib.distca_ca_fwd(None, None, None, None, None, None, None, None, ctypes.byref(_p(num_tasks=0, total_q=0, total_k=0)), None, 0, None) == 0
+
+
+def test_python_wrappers_reject_wrong_inputs():
+    """The host layer raises RuntimeError for what the reference's C++ wrappers check
+    (all_to_all.cpp:18-21, 47-99): device, rank, dtype of metadata."""
+    import torch
+    from distca_amd import ops
+    from distca_amd.fused_comm_attn import ca_varlen_fwd
+    t = torch.zeros((4, 8), dtype=torch.bfloat16)
+    off = torch.zeros(1, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="buffer"):
+        ops.a2a_memcpy_non_cp(t, off, off, True)
+    with pytest.raises(RuntimeError):
+        ops.a2a_memcpy_non_cp(t, off.to(torch.int32), off, True, buffer=torch.zeros(64, dtype=torch.uint8))
+    with pytest.raises(RuntimeError):
+        ops.pre_a2a_grad_acc(t.to(torch.float64), off.to(torch.int32), off.reshape(1, 1), off)
+    q = torch.zeros((4, 2, 128), dtype=torch.bfloat16)
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ca_varlen_fwd(q, q, q, cu, cu, 4, 4)

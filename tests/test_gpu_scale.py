@@ -198,3 +198,87 @@ def test_pack_round_trip_full_size(cuda):
         assert torch.equal(back.view(torch.int16), src.view(torch.int16))
         # a checksum of the buffer equals the checksum of the source: every byte landed exactly once
         assert int(buf.view(torch.int16).to(torch.int64).sum()) == int(src.view(torch.int16).to(torch.int64).sum())
+
+
+def test_config3_shared_kv_tasks_sampled_rows(cuda):
+    """CA tasks cut from long documents whose K/V is stored once and shared through kv_task_offsets
+    (config 3, both variants, at a quarter of the full size): sampled rows of out, lse and dq
+    against the oracle; dK/dV against the sum over tasks through <K,dK> = <Q,dQ> per document."""
+    from distca_amd import workloads
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    for variant in ("a", "b"):
+        b = workloads.config3_ca_tasks(variant=variant, total_q=65536, num_docs=4, max_doc=131072)
+        q, k, v, do, cu_q, cu_k = _dev_inputs(b, 32, 8, cuda, 60)
+        kv_off = torch.tensor(b.kv_task_offsets, dtype=torch.int32, device=cuda)
+        mq, mk = int(max(b.q_lens)), int(max(b.k_lens))
+        print(f"cfg3{variant}: {len(b.q_lens)} tasks, kv rows {b.kv_rows}", flush=True)
+        out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+        dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+        torch.cuda.synchronize()
+        rng = np.random.default_rng(1)
+        for t in rng.choice(len(b.q_lens), size=4, replace=False):
+            lq, lk = int(b.q_lens[t]), int(b.k_lens[t])
+            r0 = int(rng.integers(0, lq - 8)); r1 = r0 + 8
+            q0 = int(b.cu_seqlens_q[t]); k0 = int(b.kv_task_offsets[t])
+            kvis = r1 + (lk - lq)                         # keys beyond the last sampled row's horizon are masked anyway
+            o_ref, l_ref, dq_ref = ca_reference_rows(q[q0:q0 + r1].cpu(), k[k0:k0 + kvis].cpu(), v[k0:k0 + kvis].cpu(), do[q0:q0 + r1].cpu(),
+                                                     [0, r1], [0, kvis], 0, r0, r1, out_rows=out[q0 + r0:q0 + r1].cpu(),
+                                                     lse_rows=lse[:, q0 + r0:q0 + r1].cpu())
+            print(f"  task {t}: rows [{r0},{r1}) of {lq}, prefix {lk}", flush=True)
+            assert_close_bf16(out[q0 + r0:q0 + r1], o_ref, f"out task {t}")
+            assert (lse[:, q0 + r0:q0 + r1].cpu() - l_ref).abs().max().item() <= 2e-3
+            assert_close_bf16(dq[q0 + r0:q0 + r1], dq_ref, f"dq task {t}")
+        # scale invariance over the whole batch per kv head: sum <Q,dQ> = sum <K,dK>, sum <V,dV> = sum <O,dO>
+        whole_q, whole_k = [0, b.total_q], [0, b.kv_rows]
+        assert_identity(task_sums(q, dq, whole_q, 8), task_sums(k, dk, whole_k, 8), "<Q,dQ> = <K,dK>")
+        assert_identity(task_sums(v, dv, whole_k, 8), task_sums(out, do, whole_q, 8), "<V,dV> = <O,dO>")
+
+
+def test_ops_replay_from_a_captured_graph(cuda):
+    """Every entry point only enqueues work on the caller's stream (no allocation, no host
+    synchronisation), so a tick can be captured once and replayed.  The replays run with other
+    eager work in between and with changed inputs, and must match eager results each time."""
+    from distca_amd import workloads
+    from distca_amd._lib import CaParams, load
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    from distca_amd.ops import a2a_memcpy_non_cp
+    import ctypes
+    lens = [300, 45, 700]
+    T, hq, hkv = sum(lens), 8, 2
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=cuda)
+    g = torch.Generator(device=cuda).manual_seed(3)
+    rnd = lambda *s: torch.randn(s, generator=g, device=cuda).to(torch.bfloat16)
+    q, k, v, do = rnd(T, hq, 128), rnd(T, hkv, 128), rnd(T, hkv, 128), rnd(T, hq, 128)
+    out, lse = torch.empty_like(q), torch.empty((hq, T), dtype=torch.float32, device=cuda)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    p = CaParams(3, T, T, hq, hkv, 128, 700, 700, 128 ** -0.5, 1, 0, 0)
+    ws = torch.empty(load().distca_ca_bwd_workspace_bytes(ctypes.byref(p)), dtype=torch.uint8, device=cuda)
+    shard = torch.tensor(lens, dtype=torch.int64, device=cuda)
+    tb = hq * 256
+    off = torch.tensor([T * tb + 4096, 0, 45 * tb + 1024], dtype=torch.int64, device=cuda)  # shards out of order, with gaps
+    buf = torch.zeros(4 * T * hq * 256, dtype=torch.uint8, device=cuda)
+
+    def tick():
+        o, l = ca_varlen_fwd(q, k, v, cu, cu, 700, 700, workspace=ws)
+        out.copy_(o); lse.copy_(l)
+        ca_varlen_bwd(do, q, k, v, out, lse, cu, cu, 700, 700, dq=dq, dk=dk, dv=dv, workspace=ws)
+        a2a_memcpy_non_cp(dq.reshape(T, -1), off, shard, True, buffer=buf)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        tick()                                      # warm-up outside capture (lazy module loading)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            tick()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        q.copy_(rnd(T, hq, 128)); do.copy_(rnd(T, hq, 128))          # eager work between replays, new inputs
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (out, lse, dq, dk, dv, buf)]
+        tick()                                                        # the same tick, eagerly
+        torch.cuda.synchronize()
+        for name, a_, b_ in zip(("out", "lse", "dq", "dk", "dv", "buf"), got, (out, lse, dq, dk, dv, buf)):
+            assert torch.equal(a_, b_), f"replay {rep}: {name} differs from the eager result"
