@@ -354,8 +354,8 @@ def post_a2a_attn_out_with_lse(recv_buffer: Tensor, q: Tensor, num_heads_q: int,
     (fused_comm_attn.py:468-506): unpack the [out | lse | pad] tokens of the reply and split them.
     Returns (attn_out [T, 1, Hq*D] in q's dtype, softmax_lse_bytes [T, Hq*4] uint8)."""
     dtype = dtype or q.dtype
-    recv_shape = tuple(metadata.tensor_shape[0].recv_shape)
-    recv = torch.empty(recv_shape, dtype=torch.uint8, device=recv_buffer.device)
+    recv_shape = tuple(metadata.tensor_shape[0].recv_shape)    # in elements of `dtype`, as the reference has it
+    recv = torch.empty(recv_shape, dtype=dtype, device=recv_buffer.device).view(torch.uint8)
     post_a2a_attn_out(recv, metadata.seq_lens[0].recv_seqlens, *metadata.recv_memcpy_metadata, buffer=recv_buffer)
     itemsize = torch.empty((), dtype=dtype).element_size()
     hidden_bytes = int(q.numel() // q.shape[0]) * itemsize

@@ -12,7 +12,7 @@ document attends to the document's first i+1 shards, compute_metadata.py:404-448
 K/V shard entries with their main-copy mask and duplicate-gradient metadata (:202-219,
 277-323), and contiguous byte offsets for the q | k | v regions of each buffer.  The
 reference derives the same quantities for any number of ranks from planner output
-(_from_planner_output, :368-639); the multi-rank offset assignment is outside this build.
+(_from_planner_output, :368-639); distca_amd.compute_metadata does that.
 """
 from __future__ import annotations
 
@@ -341,7 +341,7 @@ def single_rank_step_params(plan: SingleRankPlan) -> PingPangSingleStepPackedSeq
         send = (q_off, k_off[first].unsqueeze(0), v_off[first].unsqueeze(0))      # K/V as [cp = 1, shard]
         recv = (q_off, k_off, v_off)
         seq = (SeqLens(plan.q_seqlens, plan.q_seqlens), SeqLens(stored, plan.kv_entry_tokens))
-        q_cols = qb // plan.itemsize if not backward_request else qb
+        q_cols = qb // plan.itemsize
         shape = (LogicalShape(torch.Size((tq, q_cols)), torch.Size((tq, q_cols))),
                  LogicalShape(torch.Size((1, int(stored.sum()), hkv_d)), torch.Size((tkv, hkv_d))))
         return AlltoAllMetadata((t64(0), t64(total), t64(0), t64(total)), send, recv, 0, 0, total, seq, shape,
@@ -360,7 +360,8 @@ def single_rank_step_params(plan: SingleRankPlan) -> PingPangSingleStepPackedSeq
     def out_md():
         off, _, _, total = plan.reply_layout(False)
         seq = (SeqLens(plan.q_seqlens, plan.q_seqlens),)
-        shape = (LogicalShape(torch.Size((tq, plan.out_lse_bytes)), torch.Size((tq, plan.out_lse_bytes))),)
+        cols = plan.out_lse_bytes // plan.itemsize
+        shape = (LogicalShape(torch.Size((tq, cols)), torch.Size((tq, cols))),)
         return AlltoAllMetadata((t64(0), t64(total), t64(0), t64(total)), (off,), (off,), 0, 0, total, seq, shape)
 
     attn = get_attn_metadata(plan.q_seqlens, plan.kv_seqlens)

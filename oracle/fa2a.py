@@ -26,7 +26,7 @@ import torch
 
 def _bytes2d(t: np.ndarray) -> np.ndarray:
     assert t.flags["C_CONTIGUOUS"]
-    return t.view(np.uint8).reshape(t.shape[0], -1)
+    return t.view(np.uint8).reshape(t.shape[0], int(np.prod(t.shape[1:])) * t.itemsize)
 
 
 def copy_non_cp(tensor: np.ndarray, buffer: np.ndarray, seq_offset, seq_tokens, copy_seq_mask=None,
@@ -85,7 +85,7 @@ def copy_cp(tensor: np.ndarray, buffer: np.ndarray, do_shard, seq_offset, seq_to
         tb = _bytes2d(tensor)
         num_tokens = tb.shape[0]
     else:
-        tb = tensor.view(np.uint8).reshape(tensor.shape[0] * tensor.shape[1], -1)
+        tb = tensor.view(np.uint8).reshape(tensor.shape[0] * tensor.shape[1], int(np.prod(tensor.shape[2:])) * tensor.itemsize)
         num_tokens = tensor.shape[1]
     token_bytes = tb.shape[1]
     logical_total = num_tokens * max_cp
