@@ -156,6 +156,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     l_run[m] = 0.f;
   }
   const float c = a.scale * kLog2e;
+  constexpr float kLazy = 8.f, kRedo = 32.f * 256.f;
 
   // LDS read offsets (bytes) that do not depend on the tile
   const int k_rd = l32 * kRowB + ((g ^ tile_swz(l32)) << 4);  // + kb*32*kRowB, ^ 32*s
@@ -212,40 +213,54 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     }
 #pragma unroll
     for (int m = 0; m < MSUB; ++m) {
-      float mx = sacc[m][0][0];
+      // P = 2^(S c + mc) as bf16 B operand; returns this lane's share of the row sums
+      auto exp_tile = [&](float mc) __attribute__((always_inline)) {
+        float sum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int t = 0; t < 4; ++t) {
+          const int kb = t >> 1, r0 = 8 * (t & 1);
+          float e[8];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, sacc[m][kb][r]);
-      mx = pair_max(mx);
-      const float m_new = __builtin_fmaxf(m_run[m], mx);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      if (__any(m_new != m_run[m])) {
-        const float alpha = fast_exp2((m_run[m] - m_use) * c);
-        l_run[m] *= alpha;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[m][db][r] *= alpha;
-        m_run[m] = m_new;
-      }
-      const float mc = -m_use * c;
-      float sum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, mc));
-          sacc[m][kb][r] = p;
-          sum += p;
+          for (int i = 0; i < 8; ++i) {
+            e[i] = fast_exp2(__builtin_fmaf(sacc[m][kb][r0 + i], c, mc));
+            sum += e[i];
+          }
+          pf[m][t] = cvt8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
         }
-      l_run[m] += sum;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int kb = t >> 1, r0 = 8 * (t & 1);
-        pf[m][t] = cvt8(sacc[m][kb][r0], sacc[m][kb][r0 + 1], sacc[m][kb][r0 + 2], sacc[m][kb][r0 + 3], sacc[m][kb][r0 + 4],
-                        sacc[m][kb][r0 + 5], sacc[m][kb][r0 + 6], sacc[m][kb][r0 + 7]);
+        return sum;
+      };
+      // The running reference m_run of a row need not be its maximum: any value within 2^kLazy of
+      // it gives the same O / l.  So first try the tile against the old reference, without looking
+      // for the maximum at all; only when a lane's 32 exponentials add up to more than 32 * 2^kLazy
+      // (or the row has no reference yet) is the maximum taken, the row rescaled if it moved by
+      // more than 2^kLazy, and the tile done again.
+      bool exact = __any(m_run[m] == -INFINITY);
+      float sum = 0.f;
+      if (!exact) {
+        sum = exp_tile(-m_run[m] * c);
+        exact = __any(sum > kRedo);
       }
+      if (exact) {
+        float mx = sacc[m][0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, sacc[m][kb][r]);
+        mx = pair_max(mx);
+        const float m_new = __builtin_fmaxf(m_run[m], mx);
+        if (__any((m_new - m_run[m]) * c > kLazy)) {
+          const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+          const float alpha = fast_exp2((m_run[m] - m_use) * c);
+          l_run[m] *= alpha;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[m][db][r] *= alpha;
+          m_run[m] = m_new;
+        }
+        sum = exp_tile((m_run[m] == -INFINITY) ? 0.f : -m_run[m] * c);
+      }
+      l_run[m] += sum;
     }
   };
   // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys

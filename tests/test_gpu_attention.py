@@ -77,3 +77,35 @@ def test_non_causal(cuda):
 
 def test_empty_task(cuda):
     _run([128, 0, 70], [128, 0, 70], 4, 2, 8, cuda)
+
+
+@pytest.mark.parametrize("span", [6.0, 40.0, 400.0, -400.0])
+def test_scores_that_drift_along_the_keys(cuda, span):
+    """The forward keeps a running reference per row that trails the row maximum by up to 2^8 and
+    is only corrected when a tile overshoots it.  Scores here carry a trend of `span` (natural-log
+    units) from the first key to the last: a reference that is seldom, sometimes, or in every tile
+    overtaken, and one that is never overtaken after the first tile."""
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    n, hq, hkv, d = 2048, 4, 2, 128
+    q, k, v, do = make_qkv(n, n, hq, hkv, d, 21)
+    q, k = q.float(), k.float()
+    q[:, :, 0] = 16.0
+    k[:, :, 0] = (span * (d ** 0.5) / 16.0) * torch.arange(n, dtype=torch.float32)[:, None] / n
+    q, k = q.to(torch.bfloat16), k.to(torch.bfloat16)
+    cu_q = cu([n])
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_q, cu_q)
+    dcu = torch.tensor(cu_q, device=cuda)
+    qd, kd, vd, dod = q.to(cuda), k.to(cuda), v.to(cuda), do.to(cuda)
+    print(f"case drift span={span}", flush=True)
+    out, lse = ca_varlen_fwd(qd, kd, vd, dcu, dcu, n, n, None, True, None)
+    torch.cuda.synchronize()
+    assert_close_bf16(out, ref_out, "out")
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3 * max(1.0, abs(span) / 40), "lse"
+    if abs(span) > 10:
+        return  # the backward keeps no running reference, and K entries of tens amplify the bf16 rounding of dS beyond the bar
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_q, cu_q, out=out.cpu(), softmax_lse=lse.cpu())
+    dq, dk, dv = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dcu, dcu, n, n, None, True, False, None)
+    torch.cuda.synchronize()
+    assert_close_bf16(dq, ref_dq, "dq")
+    assert_close_bf16(dk, ref_dk, "dk")
+    assert_close_bf16(dv, ref_dv, "dv")
