@@ -29,18 +29,33 @@ def _plan(seed, world, docs, max_shards, lo, hi):
 
 @pytest.mark.parametrize("seed,world,docs,max_shards,lo,hi", [(11, 3, 5, 4, 40, 300), (12, 4, 6, 5, 1, 130), (13, 2, 3, 3, 500, 1500)])
 def test_layer_step_of_several_ranks(cuda, seed, world, docs, max_shards, lo, hi):
+    _layer_step(cuda, world, _plan(seed, world, docs, max_shards, lo, hi), seed, replicas=True)
+
+
+def test_layer_step_of_a_planned_batch(cuda):
+    """The plan comes from the planner: four ranks, one of them with a long document whose middle
+    layers are handed to the others."""
+    from distca_amd.planner import PlannerConfig, plan_cost_per_rank, plan_documents
+    docs = [[2600, 300], [420], [150, 90, 64], [700]]
+    plan, load = plan_documents(docs, PlannerConfig(tolerance=0.02))
+    assert plan_cost_per_rank(plan, 4) == load and max(load) < 1.1 * sum(load) / 4
+    assert len(plan[0]) >= 5, "the long document is cut into nested layers"
+    _layer_step(cuda, 4, plan, 14, replicas=True)
+
+
+def _layer_step(cuda, world, plan, seed, replicas):
     from distca_amd.compute_metadata import from_planner_output, simulate_fa2a, step_params
     from distca_amd.dispatch_fn import pre_all2all_layout_transfer, pre_all2all_layout_transfer_backward
     from distca_amd.fused_comm_attn import (FlashAttnArgs, fused_comm_attn_backward, fused_comm_attn_forward,
                                             post_a2a_attn_out_with_lse, post_a2a_attn_out_with_lse_backward)
     hq, hkv, d = 8, 2, 128
-    plan = _plan(seed, world, docs, max_shards, lo, hi)
     lse_elems = math.ceil(hq * 4 / 16) * 16 // 2
     md = from_planner_output(world, plan, hq * d, hkv * d, lse_elems, 2, is_pipeline_tick=False, is_resend_qkv=True)
     qkv_fwd, qkv_grad, out_fwd, request, attn = md
     assert all(a["max_seqlen_q"] > 0 for a in attn), "every rank of this plan serves attention"
-    assert qkv_fwd.max_cp_degree > 1, "some K/V shard of this plan is needed on several ranks"
-    assert any(int(x.num_copies.sum()) > 0 for x in qkv_grad.kv_grad_send_dedup), "some shard is needed twice on one rank"
+    if replicas:
+        assert qkv_fwd.max_cp_degree > 1, "some K/V shard of this plan is needed on several ranks"
+        assert any(int(x.num_copies.sum()) > 0 for x in qkv_grad.kv_grad_send_dedup), "some shard is needed twice on one rank"
     steps = [step_params(r, md, cuda) for r in range(world)]
     fa_args = FlashAttnArgs(hq, hkv, d)
 
