@@ -109,3 +109,25 @@ def test_scores_that_drift_along_the_keys(cuda, span):
     assert_close_bf16(dq, ref_dq, "dq")
     assert_close_bf16(dk, ref_dk, "dk")
     assert_close_bf16(dv, ref_dv, "dv")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_task_batches(cuda, seed):
+    """Seeded random batches of CA tasks: lengths around the tile edges (32, 64, 128, 256 +- 1), prefixes
+    longer than the query shard, every head grouping the kernels accept, causal or not, with and
+    without tasks that share one stored K/V copy."""
+    rng = np.random.default_rng(1000 + seed)
+    edges = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 383, 511, 513]
+    n = int(rng.integers(1, 7))
+    q_lens = [int(rng.choice(edges)) if rng.random() < 0.7 else int(rng.integers(1, 700)) for _ in range(n)]
+    if rng.random() < 0.25:
+        q_lens[int(rng.integers(n))] = 0
+    hq, hkv = [(4, 4), (8, 2), (8, 1), (12, 4), (16, 2), (2, 1)][int(rng.integers(6))]
+    causal = bool(rng.random() < 0.8)
+    if rng.random() < 0.3 and all(q_lens):
+        # shards of one document over one stored copy of its K/V
+        ends = np.cumsum(q_lens)
+        _run(q_lens, [int(e) for e in ends], hq, hkv, seed, cuda, causal=causal, kv_offsets=[0] * n, total_k=int(ends[-1]))
+        return
+    k_lens = [q + (int(rng.choice(edges)) if (q and rng.random() < 0.5) else 0) for q in q_lens]
+    _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=causal)
