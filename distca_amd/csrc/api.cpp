@@ -1,6 +1,7 @@
 // Process-wide state behind the C ABI: error text and device facts.
 #include "api_util.h"
 
+#include <atomic>
 #include <utility>
 #include <vector>
 
@@ -21,6 +22,13 @@ int num_compute_units() {
     cached[dev] = n;
   }
   return cached[dev];
+}
+
+bool first_use_on_this_device(int slot) {
+  static std::atomic<unsigned char> seen[64][kSlotCount];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || slot < 0 || slot >= kSlotCount) return true;
+  return seen[dev][slot].exchange(1) == 0;
 }
 
 namespace {

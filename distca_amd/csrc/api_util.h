@@ -39,5 +39,9 @@ struct ScopedTimer {
 
 // Number of compute units of the current device (cached per device id).
 int num_compute_units();
+// True the first time it is called with `slot` on the current device: per-device set-up such as
+// raising a kernel's dynamic LDS limit is done once for each GPU the library runs on.
+bool first_use_on_this_device(int slot);
+enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotCount = 2 };
 
 }  // namespace distca

@@ -753,13 +753,11 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   if ((uint64_t)p->max_seqlen_q * a.group * a.group >= (1ull << 32))
     return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: max_seqlen_q * (Hq/Hkv)^2 must stay below 2^32");
 
-  static bool attr_set = false;
-  if (!attr_set) {
+  if (first_use_on_this_device(kSlotBwdLds)) {
     hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
     hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
     hipError_t e3 = hipFuncSetAttribute((const void *)ca_bwd_dq_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
     if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve LDS");
-    attr_set = true;
   }
 
   // ---- dK, dV: one workgroup per (task, 128-key block, kv head)

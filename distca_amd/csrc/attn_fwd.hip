@@ -390,11 +390,9 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   const int64_t grid = max_items * p->num_heads_kv;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
-  static bool attr_set = false;
-  if (!attr_set) {
+  if (first_use_on_this_device(kSlotFwdLds)) {
     hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
     if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
-    attr_set = true;
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);
