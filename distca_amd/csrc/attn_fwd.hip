@@ -48,6 +48,11 @@ struct FwdArgs {
   int32_t hq, hkv, group, total_q;
   int32_t causal;
   float scale;
+  // Where the query and output tokens live.  Token t of task b starts at base + off[b] + t * tok_bytes
+  // (off == nullptr: the packed tensor, off[b] = cu_q[b] * tok_bytes); head h at + h * 256 bytes.
+  const int64_t *q_task_off, *out_task_off;
+  int64_t q_tok_bytes, out_tok_bytes;
+  int32_t lse_in_token;  // 1: lse of (token, head) as fp32 at token + hq * 256 + h * 4 (the [out | lse] reply), 0: lse[h][token]
 };
 
 template <int MSUB>
@@ -81,6 +86,8 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int ntiles = nvis > 0 ? (nvis + kFwdKV - 1) / kFwdKV : 0;
 
   // ---- per-lane rows
+  const uint8_t *qbytes = reinterpret_cast<const uint8_t *>(a.q) + (a.q_task_off ? a.q_task_off[task] : (int64_t)q0 * a.q_tok_bytes);
+  uint8_t *obytes = reinterpret_cast<uint8_t *>(a.out) + (a.out_task_off ? a.out_task_off[task] : (int64_t)q0 * a.out_tok_bytes);
   int row[MSUB], tok[MSUB], lim[MSUB];
   bool valid[MSUB];
   const __bf16 *qptr[MSUB];
@@ -93,7 +100,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     int lm = a.causal ? tok[m] + shift : lk - 1;
     if (lm > lk - 1) lm = lk - 1;
     lim[m] = lm;
-    qptr[m] = a.q + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+    qptr[m] = reinterpret_cast<const __bf16 *>(qbytes + (int64_t)tok[m] * a.q_tok_bytes) + (kvh * G + hg) * kHeadDim;
   }
   // wave-uniform limits: first row's limit decides whether a tile needs masking, last row's
   // whether the wave has anything to do in it.
@@ -330,7 +337,8 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
-      __bf16 *op = a.out + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+      uint8_t *otok = obytes + (int64_t)tok[m] * a.out_tok_bytes;
+      __bf16 *op = reinterpret_cast<__bf16 *>(otok) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -343,7 +351,16 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
         }
       if (g == 0) {
         const float lse = l_tot > 0.f ? (m_run[m] * c + fast_log2(l_tot)) * kLn2 : -INFINITY;
-        a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]] = lse;
+        const int head = kvh * G + hg;
+        if (a.lse_in_token) {
+          float *lp = reinterpret_cast<float *>(otok + (int64_t)a.hq * kHeadDim * 2);
+          lp[head] = lse;
+          if (head == a.hq - 1) {  // zero the padding that rounds the token up to 16 bytes
+            for (int64_t b = (int64_t)a.hq * (kHeadDim * 2 + 4); b < (((int64_t)a.hq * (kHeadDim * 2 + 4) + 15) & ~(int64_t)15); b += 4) *reinterpret_cast<float *>(otok + b) = 0.f;
+          }
+        } else {
+          a.lse[(int64_t)head * a.total_q + q0 + tok[m]] = lse;
+        }
       }
     }
   }
@@ -361,15 +378,37 @@ extern "C" int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p) {
   return sched_region_bytes(p->num_tasks, fwd_max_items(p));
 }
 
+extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,
+                                    const void *v, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes,
+                                    float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
+                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+
 extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
                              int64_t workspace_bytes, void *stream) {
+  if (!lse) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
+  return distca_ca_fwd_tokens(q, nullptr, 0, k, v, out, nullptr, 0, lse, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+}
+
+extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,
+                                    const void *v, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes,
+                                    float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
+                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  const void *q = q_base;
+  void *out = out_base;
   if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
   int rc = validate_params(p);
   if (rc) return rc;
   if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
-  if (!q || !k || !v || !out || !lse || !cu_q || !cu_k) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
+  if (!q || !k || !v || !out || !cu_q || !cu_k) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return fail(DISTCA_E_INVALID, "ca_fwd: q/k/v/out must be 16-byte aligned");
+  const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2;
+  if (!q_task_off) q_tok_bytes = row_bytes;
+  if (!out_task_off) out_tok_bytes = row_bytes;
+  if (q_tok_bytes < row_bytes || (q_tok_bytes & 15)) return fail(DISTCA_E_INVALID, "ca_fwd: query token of %lld B (needs >= %lld, multiple of 16)", (long long)q_tok_bytes, (long long)row_bytes);
+  const int64_t out_need = row_bytes + (lse ? 0 : (int64_t)p->num_heads_q * 4);
+  if (out_tok_bytes < out_need || (out_tok_bytes & 15)) return fail(DISTCA_E_INVALID, "ca_fwd: output token of %lld B (needs >= %lld, multiple of 16)", (long long)out_tok_bytes, (long long)out_need);
+  if (!lse && !out_task_off) return fail(DISTCA_E_INVALID, "ca_fwd: lse is null and the output is not in token layout");
   const int64_t need = distca_ca_fwd_workspace_bytes(p);
   if (!workspace || workspace_bytes < need) return fail(DISTCA_E_WORKSPACE, "ca_fwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)need);
   if (!aligned16(workspace)) return fail(DISTCA_E_INVALID, "ca_fwd: workspace must be 16-byte aligned");
@@ -388,6 +427,8 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
+  a.q_task_off = q_task_off; a.out_task_off = out_task_off; a.q_tok_bytes = q_tok_bytes; a.out_tok_bytes = out_tok_bytes;
+  a.lse_in_token = lse ? 0 : 1;
   const int64_t grid = max_items * p->num_heads_kv;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
   if (first_use_on_this_device(kSlotFwdLds)) {

@@ -17,6 +17,8 @@ import torch
 from torch import Tensor
 
 from . import _lib
+from .ops import a2a_memcpy_non_cp
+from .utils import size_pad_by_int4
 from .dispatch import (post_a2a_attn_out, post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_grad_resend_qkv,
                        pre_a2a_attn_out_with_lse, pre_a2a_qkv)
 
@@ -255,13 +257,48 @@ class ServerFwdMeta:
 
 
 def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdMeta, fa_params: PackedSeqParams,
-                      fa_args: FlashAttnArgs, dtype: torch.dtype = torch.bfloat16):
+                      fa_args: FlashAttnArgs, dtype: torch.dtype = torch.bfloat16, in_place: bool = True):
     """fused_comm_attn.py:298-389: unpack q,k,v -> attention -> pack [out | lse].
-    Returns (attn_out [T,Hq*D], softmax_lse [Hq,T]) as well, for the caller's own use."""
+
+    With `in_place` (the default) the kernel reads the query tokens where they lie in the receive
+    buffer and writes the [out | lse] tokens where they belong in the send buffer; only K and V are
+    unpacked (a shard read by several tasks is copied once per task).  Returns (None, None) then.
+    Without it every step is its own pass, as in the reference, and (attn_out [T,Hq*D],
+    softmax_lse [Hq,T]) are returned for the caller's own use.  Both leave the same bytes in the
+    send buffer."""
     dev = recv_buffer.device
-    recv_q = torch.empty(meta.recv_q_shape, dtype=dtype, device=dev)
     recv_k = torch.empty(meta.recv_k_shape, dtype=dtype, device=dev)
     recv_v = torch.empty_like(recv_k)
+    hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
+    if in_place and dtype == torch.bfloat16:
+        a2a_memcpy_non_cp(recv_k, meta.k_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
+        a2a_memcpy_non_cp(recv_v, meta.v_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
+        tq, tk = int(meta.recv_q_shape[0]), int(meta.recv_k_shape[0])
+        scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
+        lib = _lib.load()
+        cu_q, cu_k = fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv
+        kv_off = getattr(fa_params, "kv_task_offsets", None)
+        assert fa_args.causal and fa_args.window_size == (-1, -1) and fa_args.dropout_p == 0.0
+        p = _params(cu_q.shape[0] - 1, tq, tk, hq, hkv, d, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, scale,
+                    fa_args.causal, False)
+        need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
+        if need < 0:
+            _lib.check(int(need), "ca_server_forward")
+        ws = _workspace(None, int(need), dev)
+        q_tok = hq * d * 2
+        out_tok = size_pad_by_int4(q_tok + hq * 4, 1)[0]
+        for name, t in (("q_recv_offset", meta.q_recv_offset), ("out_send_offset", meta.out_send_offset)):
+            if t.dtype != torch.int64 or not t.is_cuda or t.numel() != cu_q.shape[0] - 1:
+                raise RuntimeError(f"{name} must be an int64 CUDA tensor with one entry per task")
+        with torch.cuda.device(dev):
+            rc = lib.distca_ca_fwd_tokens(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), q_tok, recv_k.data_ptr(),
+                                          recv_v.data_ptr(), send_buffer.data_ptr(), meta.out_send_offset.data_ptr(), out_tok,
+                                          None, cu_q.data_ptr(), cu_k.data_ptr(), kv_off.data_ptr() if kv_off is not None else None,
+                                          ctypes.byref(p), ws.data_ptr(),
+                                          ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "ca_server_forward")
+        return None, None
+    recv_q = torch.empty(meta.recv_q_shape, dtype=dtype, device=dev)
     post_a2a_qkv(recv_q, recv_k, recv_v, None, meta.q_recv_seq_tokens, meta.k_recv_seq_tokens,
                  meta.q_recv_offset, meta.k_recv_offset, meta.v_recv_offset, is_fwd=True, buffer=recv_buffer)
     attn_out, softmax_lse = _qkv_to_attn_out_fwd(recv_q, recv_k, recv_v, fa_params, fa_args)

@@ -129,6 +129,28 @@ int distca_ca_fwd(const void *q, const void *k, const void *v, void *out,
                   const distca_ca_params *p, void *workspace,
                   int64_t workspace_bytes, void *stream);
 
+/* The same forward with the query and output tokens where the CA server has them
+ * (distca/runtime/megatron/ops/fused_comm_attn.py:298-389 unpacks q from the
+ * receive buffer, runs attention, and packs [out | lse] tokens into the send
+ * buffer, attn_kernels/dispatch.py:209-221; here the kernel reads and writes
+ * those tokens in place).  Token t of task b of the queries starts at
+ * q_base + q_task_off[b] + t * q_tok_bytes and holds Hq*D bf16; of the output at
+ * out_base + out_task_off[b] + t * out_tok_bytes and receives Hq*D bf16, then,
+ * when lse is NULL, Hq fp32 lse values and zero padding up to the next multiple
+ * of 16 bytes.  A NULL offset array means the packed tensor (offset of task b =
+ * cu_seqlens_q[b] tokens, token size Hq*D*2); lse == NULL needs out_task_off.
+ * Offsets are device int64 arrays of num_tasks entries, multiples of 16; token
+ * sizes are multiples of 16.  Ranges are the caller's responsibility. */
+int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off,
+                         int64_t q_tok_bytes, const void *k, const void *v,
+                         void *out_base, const int64_t *out_task_off,
+                         int64_t out_tok_bytes, float *lse,
+                         const int32_t *cu_seqlens_q,
+                         const int32_t *cu_seqlens_k,
+                         const int32_t *kv_task_offsets,
+                         const distca_ca_params *p, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
 /* dk/dv rows are written once per task when kv_task_offsets is NULL.  When it
  * is given, tasks may alias KV rows and dk/dv hold the sum over every task
  * that read the row (what the reference obtains with duplicated KV copies and

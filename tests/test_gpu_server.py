@@ -82,8 +82,12 @@ def test_server_tick_forward_and_backward(cuda):
                          _dev(q_lens, cuda, torch.int64), _dev(so, cuda),
                          (tq, HQ * D), (sum(k_lens_shard), HKV * D))
     print("server forward", flush=True)
-    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, meta, fa_params, fa_args)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, meta, fa_params, fa_args, in_place=False)
+    # the same tick with the kernel reading q from the receive buffer and writing [out | lse] into the send buffer
+    send_in_place = torch.full_like(send, 0xCD)
+    assert ca_server_forward(torch.from_numpy(recv).to(cuda), send_in_place, meta, fa_params, fa_args) == (None, None)
     torch.cuda.synchronize()
+    assert torch.equal(send_in_place, send), "in-place and step-by-step ticks leave the same bytes"
 
     # numerics: three prefix tasks == whole-document causal attention
     cu_doc = np.array([0, 600, 730], np.int32)
@@ -201,8 +205,11 @@ def test_server_tick_from_single_rank_plan(cuda):
     fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
     send = torch.zeros(f_send, dtype=torch.uint8, device=cuda)
     print("plan forward", flush=True)
-    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args, in_place=False)
+    send_in_place = torch.zeros_like(send)
+    ca_server_forward(torch.from_numpy(recv).to(cuda), send_in_place, fmeta, fa_params, fa_args)
     torch.cuda.synchronize()
+    assert torch.equal(send_in_place, send)
     cu_doc = np.concatenate([[0], np.cumsum([sum(d) for d in docs])]).astype(np.int32)
     ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_doc, cu_doc)
     assert_close_bf16(out.reshape(T, 8, 128), ref_out, "out")
