@@ -386,6 +386,10 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
 extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
                              int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
+  const int rc = validate_params(p);
+  if (rc) return rc;
+  if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
   if (!lse) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
   return distca_ca_fwd_tokens(q, nullptr, 0, k, v, out, nullptr, 0, lse, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
 }
