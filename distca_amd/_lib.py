@@ -13,7 +13,7 @@ from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int6
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdistca_ca.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class CaParams(Structure):
@@ -41,6 +41,8 @@ SYMBOLS = {
     "distca_ca_fwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                      c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_bwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_schedule_host": (c_int64, [c_int, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64]),
     "distca_timing_enable": (None, [c_int]),
     "distca_timing_read": (c_int, [c_int, POINTER(ctypes.c_double), POINTER(c_int64)]),

@@ -79,6 +79,11 @@ struct BwdArgs {
   uint32_t group_magic;  // ceil(2^32 / group), 0 when group == 1: n / group == umulhi(n, magic) for n * group < 2^32
   int32_t causal;
   float scale;
+  // Where the query-side tokens live: q and dout point at the first byte of their part of token 0 of a
+  // region in which token t of task b starts at off[b] + t * tok_bytes (off == nullptr: the packed
+  // tensors, off[b] = cu_q[b] * tok_bytes); head h at + h * 256 bytes.  dq likewise.
+  const int64_t *qs_task_off, *dq_task_off;
+  int64_t qs_tok_bytes, dq_tok_bytes;
 };
 
 template <bool ALIAS>
@@ -145,7 +150,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       dvacc[db][r] = 0.f;
     }
 
-  const int64_t qbase = ((int64_t)q0 * a.hq + kvh * G) * kHeadDim;  // element offset of (token q0, first head of the group)
+  // byte offset of (token 0 of the task, first head of the group) in the query-side region
+  const int64_t qbase = (a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes) + (int64_t)kvh * G * kHeadDim * 2;
 
   // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block.
   // Rows past the task (and a group's last block when it does not exist) are clamped to the
@@ -183,9 +189,9 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       const int tok = div_group(ok ? rho : 0);
       const int hg = (ok ? rho : 0) - tok * G;
       const int chunk = (lane & 15) ^ tile_swz(rl);
-      const int64_t eo = qbase + (int64_t)(tok * a.hq + hg) * kHeadDim;
-      const __bf16 *qs = ok ? a.q + eo : reinterpret_cast<const __bf16 *>(a.zero_row);
-      const __bf16 *ds = ok ? a.dout + eo : reinterpret_cast<const __bf16 *>(a.zero_row);
+      const int64_t eo = qbase + (int64_t)tok * a.qs_tok_bytes + hg * (kHeadDim * 2);
+      const __bf16 *qs = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
+      const __bf16 *ds = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
       const uint32_t dst = lds0 + tile + (kbw * 8 + 4 * i) * kTileRow;
       lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
       lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
@@ -406,6 +412,8 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   const int task = it4.x, mblk = it4.y;
 
   const int q0 = a.cu_q[task];
+  const int64_t qs_task = a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes;
+  const int64_t dq_task = a.dq_task_off ? a.dq_task_off[task] : (int64_t)q0 * a.dq_tok_bytes;
   const int lq = a.cu_q[task + 1] - q0;
   const int lk = a.cu_k[task + 1] - a.cu_k[task];
   const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
@@ -437,7 +445,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     int lm = a.causal ? tok[m] + shift : lk - 1;
     if (lm > lk - 1) lm = lk - 1;
     lim[m] = lm;
-    const int64_t ro = ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim + 8 * g;
+    const int64_t ro = qs_task + (int64_t)tok[m] * a.qs_tok_bytes + ((kvh * G + hg) * kHeadDim + 8 * g) * 2;  // bytes
     lse2[m] = INFINITY;  // rows past the task: P = exp2(-inf) = 0
     dsc[m] = 0.f;
     if (valid[m]) {
@@ -448,8 +456,8 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       if (valid[m]) {
-        qf[m][s] = *reinterpret_cast<const bf16x8 *>(a.q + ro + 16 * s);
-        dof[m][s] = *reinterpret_cast<const bf16x8 *>(a.dout + ro + 16 * s);
+        qf[m][s] = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s);
+        dof[m][s] = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
       } else {
         qf[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
         dof[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -607,7 +615,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   for (int m = 0; m < MSUB; ++m) {
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
-      __bf16 *op = a.dq + ((int64_t)(q0 + tok[m]) * a.hq + kvh * G + hg) * kHeadDim;
+      __bf16 *op = reinterpret_cast<__bf16 *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -621,27 +629,47 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
 }
 
 // Per (token, head) row: dscaled[h][t] = scale * sum_d dO*O and lse2[h][t] = lse[h][t]*log2(e).
-__global__ __launch_bounds__(256) void bwd_prepare_kernel(const __bf16 *__restrict__ dout, const __bf16 *__restrict__ out,
-                                                         const float *__restrict__ lse, float *__restrict__ dscaled,
-                                                         float *__restrict__ lse2, int64_t rows, int32_t hq, int32_t total_q,
-                                                         float scale) {
+// dout and out point at their part of token 0 of a region laid out like BwdArgs' query side; lse is
+// [Hq][Tq] fp32, or, when lse_tok is given instead, Hq fp32 per token at lse_tok + token start.
+__global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restrict__ dout, const uint8_t *__restrict__ out,
+                                                         const float *__restrict__ lse, const uint8_t *__restrict__ lse_tok,
+                                                         const int64_t *__restrict__ task_off, int64_t tok_bytes,
+                                                         const int32_t *__restrict__ cu_q, int32_t num_tasks,
+                                                         float *__restrict__ dscaled, float *__restrict__ lse2, int64_t rows,
+                                                         int32_t hq, int32_t total_q, float scale) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int sub = threadIdx.x & 15;
   float s = 0.f;
+  int64_t t = 0, tok_start = 0;
+  int h = 0;
   if (row < rows) {
-    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(dout + row * kHeadDim + sub * 8);
-    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(out + row * kHeadDim + sub * 8);
+    t = row / hq;
+    h = (int)(row - t * hq);
+    if (task_off) {
+      // the task that holds token t: last b with cu_q[b] <= t
+      int lo = 0, hi = num_tasks - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (cu_q[mid] <= t) lo = mid;
+        else hi = mid - 1;
+      }
+      tok_start = task_off[lo] + (t - cu_q[lo]) * tok_bytes;
+    } else {
+      tok_start = t * tok_bytes;
+    }
+    const int64_t eo = tok_start + (int64_t)h * (kHeadDim * 2) + sub * 16;
+    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(dout + eo);
+    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(out + eo);
 #pragma unroll
     for (int i = 0; i < 8; ++i) s += (float)a[i] * (float)b[i];
   }
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
   if (row < rows && sub == 0) {
-    const int64_t t = row / hq;
-    const int h = (int)(row - t * hq);
     const int64_t o = (int64_t)h * total_q + t;
     dscaled[o] = s * scale;
-    lse2[o] = lse[o] * kLog2e;
+    const float l = lse_tok ? reinterpret_cast<const float *>(lse_tok + tok_start)[h] : lse[o];
+    lse2[o] = l * kLog2e;
   }
 }
 
@@ -698,16 +726,65 @@ extern "C" int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p) {
   return bwd_layout(p, true).total;
 }
 
+namespace {
+// The query side of a backward call: where dO, O, lse, q are read and dq is written.
+struct BwdQuerySide {
+  const void *dout, *q, *out;      // first byte of each part in token 0 of its region
+  const float *lse;                // [Hq][Tq], or nullptr with lse_tok
+  const void *lse_tok;             // first byte of the lse part in token 0, or nullptr
+  const int64_t *task_off;         // shared by dout, q, out, lse_tok; nullptr = packed tensors
+  int64_t tok_bytes;
+  void *dq;
+  const int64_t *dq_task_off;
+  int64_t dq_tok_bytes;
+};
+int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+}  // namespace
+
 extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
                              void *dq, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
                              const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
+  const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2;
+  const BwdQuerySide qs{dout, q, out, lse, nullptr, nullptr, row_bytes, dq, nullptr, row_bytes};
+  return run_bwd(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+}
+
+extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off, int64_t req_tok_bytes, const void *k,
+                                    const void *v, void *dq_base, const int64_t *dq_task_off, int64_t dq_tok_bytes, void *dk,
+                                    void *dv, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
+                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2, lse_bytes = (int64_t)p->num_heads_q * 4;
+  if (lse_bytes & 15)
+    return fail(DISTCA_E_UNSUPPORTED, "ca_bwd_tokens: %d query heads put the q part of a request token off 16-byte alignment", p->num_heads_q);
+  if (!req_task_off || !dq_task_off) return fail(DISTCA_E_INVALID, "ca_bwd_tokens: null offset array");
+  if (req_tok_bytes < 3 * row_bytes + lse_bytes || (req_tok_bytes & 15))
+    return fail(DISTCA_E_INVALID, "ca_bwd_tokens: request token of %lld B (needs >= %lld, multiple of 16)", (long long)req_tok_bytes, (long long)(3 * row_bytes + lse_bytes));
+  if (dq_tok_bytes < row_bytes || (dq_tok_bytes & 15))
+    return fail(DISTCA_E_INVALID, "ca_bwd_tokens: dq token of %lld B (needs >= %lld, multiple of 16)", (long long)dq_tok_bytes, (long long)row_bytes);
+  const uint8_t *r = (const uint8_t *)req_base;
+  // [dO | O | lse | q | pad]
+  const BwdQuerySide qs{r, r ? r + 2 * row_bytes + lse_bytes : nullptr, r ? r + row_bytes : nullptr, nullptr,
+                        r ? r + 2 * row_bytes : nullptr, req_task_off, req_tok_bytes, dq_base, dq_task_off, dq_tok_bytes};
+  return run_bwd(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+}
+
+namespace {
+int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  const void *dout = qs.dout, *q = qs.q, *out = qs.out;
+  void *dq = qs.dq;
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
   int rc = validate_params(p);
   if (rc) return rc;
   const bool alias = kv_off != nullptr;
   if (p->deterministic && alias)
     return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: deterministic=1 with kv_task_offsets (dK/dV of aliased rows are summed with float atomics)");
-  if (!dout || !q || !k || !v || !out || !lse || !dq || !dk || !dv || !cu_q || !cu_k) {
+  if (!dout || !q || !k || !v || !out || (!qs.lse && !qs.lse_tok) || !dq || !dk || !dv || !cu_q || !cu_k) {
     if (p->num_tasks == 0 || (p->total_q == 0 && p->total_k == 0)) return DISTCA_OK;
     return fail(DISTCA_E_INVALID, "ca_bwd: null pointer");
   }
@@ -735,14 +812,15 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   if (p->num_tasks == 0 || p->total_q == 0) return check_launch("ca_bwd(clear)");
 
   const int64_t rows = (int64_t)p->total_q * p->num_heads_q;
-  hipLaunchKernelGGL(bwd_prepare_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, (const __bf16 *)dout,
-                     (const __bf16 *)out, lse, (float *)(ws + w.delta), (float *)(ws + w.lse2), rows, p->num_heads_q, p->total_q,
-                     p->softmax_scale);
+  hipLaunchKernelGGL(bwd_prepare_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, (const uint8_t *)dout,
+                     (const uint8_t *)out, qs.lse, (const uint8_t *)qs.lse_tok, qs.task_off, qs.tok_bytes, cu_q, p->num_tasks,
+                     (float *)(ws + w.delta), (float *)(ws + w.lse2), rows, p->num_heads_q, p->total_q, p->softmax_scale);
 
   BwdArgs a;
   a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v; a.dout = (const __bf16 *)dout;
   a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta);
   a.dq = (__bf16 *)dq; a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
+  a.qs_task_off = qs.task_off; a.qs_tok_bytes = qs.tok_bytes; a.dq_task_off = qs.dq_task_off; a.dq_tok_bytes = qs.dq_tok_bytes;
   a.dk_acc = alias ? (float *)(ws + w.dk_acc) : nullptr;
   a.dv_acc = alias ? (float *)(ws + w.dv_acc) : nullptr;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
@@ -796,3 +874,4 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   (void)q_elems;
   return check_launch("ca_bwd");
 }
+}  // namespace

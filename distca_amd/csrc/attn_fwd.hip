@@ -406,13 +406,13 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
   if (!q || !k || !v || !out || !cu_q || !cu_k) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return fail(DISTCA_E_INVALID, "ca_fwd: q/k/v/out must be 16-byte aligned");
+  if (!lse && !out_task_off) return fail(DISTCA_E_INVALID, "ca_fwd: lse is null and the output is not in token layout");
   const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2;
   if (!q_task_off) q_tok_bytes = row_bytes;
   if (!out_task_off) out_tok_bytes = row_bytes;
   if (q_tok_bytes < row_bytes || (q_tok_bytes & 15)) return fail(DISTCA_E_INVALID, "ca_fwd: query token of %lld B (needs >= %lld, multiple of 16)", (long long)q_tok_bytes, (long long)row_bytes);
   const int64_t out_need = row_bytes + (lse ? 0 : (int64_t)p->num_heads_q * 4);
   if (out_tok_bytes < out_need || (out_tok_bytes & 15)) return fail(DISTCA_E_INVALID, "ca_fwd: output token of %lld B (needs >= %lld, multiple of 16)", (long long)out_tok_bytes, (long long)out_need);
-  if (!lse && !out_task_off) return fail(DISTCA_E_INVALID, "ca_fwd: lse is null and the output is not in token layout");
   const int64_t need = distca_ca_fwd_workspace_bytes(p);
   if (!workspace || workspace_bytes < need) return fail(DISTCA_E_WORKSPACE, "ca_fwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)need);
   if (!aligned16(workspace)) return fail(DISTCA_E_INVALID, "ca_fwd: workspace must be 16-byte aligned");

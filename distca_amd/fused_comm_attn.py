@@ -17,7 +17,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .ops import a2a_memcpy_non_cp
+from .ops import a2a_memcpy_non_cp, pre_a2a_grad_acc
 from .utils import size_pad_by_int4
 from .dispatch import (post_a2a_attn_out, post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_grad_resend_qkv,
                        pre_a2a_attn_out_with_lse, pre_a2a_qkv)
@@ -329,12 +329,48 @@ class ServerBwdMeta:
 
 def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwdMeta, fa_args: FlashAttnArgs,
                        cu_seqlens_q: Tensor, cu_seqlens_kv: Tensor, max_seqlen_q: int, max_seqlen_kv: int,
-                       dtype: torch.dtype = torch.bfloat16):
+                       dtype: torch.dtype = torch.bfloat16, in_place: bool = True):
     """fused_comm_attn.py:407-461: unpack merged request -> attention backward -> sum
-    duplicate KV gradients -> masked pack of dq, dk, dv."""
+    duplicate KV gradients -> masked pack of dq, dk, dv.
+
+    With `in_place` (the default, for head counts that keep the q part of a request token 16-byte
+    aligned) the kernels read dO, O, lse and q where they lie in the receive buffer and write dq
+    where it belongs in the send buffer; K and V are unpacked, dk and dv summed and packed as
+    before.  Returns (None, dk, dv) then, else (dq, dk, dv).  Both leave the same bytes in the send
+    buffer."""
     dev = recv_buffer.device
     recv_k = torch.empty(meta.k_shape, dtype=dtype, device=dev)
     recv_v = torch.empty_like(recv_k)
+    hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
+    if in_place and (hq * 4) % 16 == 0 and dtype == torch.bfloat16:
+        a2a_memcpy_non_cp(recv_k, meta.k_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
+        a2a_memcpy_non_cp(recv_v, meta.v_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
+        tq, tk = int(meta.attn_out_shape[0]), int(meta.k_shape[0])
+        scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
+        lib = _lib.load()
+        p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_kv, scale, fa_args.causal,
+                    fa_args.deterministic)
+        need = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+        if need < 0:
+            _lib.check(int(need), "ca_server_backward")
+        ws = _workspace(None, int(need), dev)
+        row = hq * d * 2
+        req_tok = size_pad_by_int4(3 * row + hq * 4, 1)[0]
+        for name, t in (("q_recv_offset", meta.q_recv_offset), ("q_grad_send_offset", meta.q_grad_send_offset)):
+            if t.dtype != torch.int64 or not t.is_cuda or t.numel() != cu_seqlens_q.shape[0] - 1:
+                raise RuntimeError(f"{name} must be an int64 CUDA tensor with one entry per task")
+        dk = torch.empty((tk, hkv * d), dtype=dtype, device=dev)
+        dv = torch.empty_like(dk)
+        with torch.cuda.device(dev):
+            rc = lib.distca_ca_bwd_tokens(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), req_tok, recv_k.data_ptr(),
+                                          recv_v.data_ptr(), send_buffer.data_ptr(), meta.q_grad_send_offset.data_ptr(), row,
+                                          dk.data_ptr(), dv.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_kv.data_ptr(), None,
+                                          ctypes.byref(p), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "ca_server_backward")
+        for g, off in ((dk, meta.k_grad_send_offset), (dv, meta.v_grad_send_offset)):
+            pre_a2a_grad_acc(g, meta.num_copies, meta.copy_start_id, meta.k_grad_send_seq_tokens)
+            a2a_memcpy_non_cp(g, off, meta.k_grad_send_seq_tokens, True, shard_do_copy_mask=meta.main_copy_mask, buffer=send_buffer)
+        return None, dk, dv
     (dout, out, lse, q, recv_k, recv_v) = post_a2a_attn_out_grad_resend_qkv(
         meta.attn_out_shape, meta.lse_shape, meta.attn_out_shape, torch.float32, recv_k, recv_v, None,
         meta.q_recv_seq_tokens, meta.k_recv_seq_tokens, meta.q_recv_offset, meta.k_recv_offset, meta.v_recv_offset,

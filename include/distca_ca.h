@@ -162,6 +162,26 @@ int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v,
                   const distca_ca_params *p, void *workspace,
                   int64_t workspace_bytes, void *stream);
 
+/* The same backward with the query side where the CA server has it
+ * (fused_comm_attn.py:407-461 unpacks the request tokens [dO | O | lse | q | pad]
+ * of attn_kernels/dispatch.py:138-206 into four tensors, runs the backward and
+ * packs dq; here the kernels read the parts of each token in place and write dq
+ * tokens into the send buffer).  Token t of task b of the request starts at
+ * req_base + req_task_off[b] + t * req_tok_bytes and holds Hq*D bf16 dO, Hq*D
+ * bf16 O, Hq fp32 lse, Hq*D bf16 q; dq token t of task b starts at
+ * dq_base + dq_task_off[b] + t * dq_tok_bytes.  Needs Hq % 4 == 0 (the q part must
+ * stay 16-byte aligned; other head counts return DISTCA_E_UNSUPPORTED and are
+ * served by distca_ca_bwd on unpacked tensors).  dk / dv as in distca_ca_bwd. */
+int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off,
+                         int64_t req_tok_bytes, const void *k, const void *v,
+                         void *dq_base, const int64_t *dq_task_off,
+                         int64_t dq_tok_bytes, void *dk, void *dv,
+                         const int32_t *cu_seqlens_q,
+                         const int32_t *cu_seqlens_k,
+                         const int32_t *kv_task_offsets,
+                         const distca_ca_params *p, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Tile scheduler, host mirror.  The device builds the same list inside
  * distca_ca_fwd / distca_ca_bwd; this entry point runs the identical code on

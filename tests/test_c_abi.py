@@ -165,3 +165,35 @@ def test_python_wrappers_reject_wrong_inputs():
     cu = torch.tensor([0, 4], dtype=torch.int32)
     with pytest.raises(RuntimeError, match="CUDA"):
         ca_varlen_fwd(q, q, q, cu, cu, 4, 4)
+
+
+def test_token_layout_entry_points_check_their_layouts():
+    """distca_ca_fwd_tokens / distca_ca_bwd_tokens refuse token sizes that cannot hold their parts, a
+    missing lse destination, and (backward) head counts that put q off 16-byte alignment; all before
+    any launch."""
+    lib = _lib.load()
+    ptr = ctypes.c_void_p(0x1000)
+    p = _lib.CaParams(2, 64, 64, 8, 2, 128, 32, 32, 0.088, 1, 0, 0)
+    need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
+    row = 8 * 128 * 2
+    fwd = lambda **kw: lib.distca_ca_fwd_tokens(*[kw.get(n, d) for n, d in (
+        ("q", ptr), ("q_off", ptr), ("q_tok", row), ("k", ptr), ("v", ptr), ("out", ptr), ("out_off", ptr), ("out_tok", row + 32),
+        ("lse", None), ("cu_q", ptr), ("cu_k", ptr), ("kv_off", None), ("p", ctypes.byref(p)), ("ws", ptr), ("ws_bytes", 16), ("stream", None))])
+    assert fwd() == -3 and b"workspace" in lib.distca_last_error()          # everything else is in order
+    assert fwd(q_tok=row - 16) == -1 and b"query token" in lib.distca_last_error()
+    assert fwd(out_tok=row) == -1 and b"output token" in lib.distca_last_error()   # no room for the lse
+    assert fwd(out_tok=row + 8) == -1
+    assert fwd(out_off=None, out_tok=0) == -1 and b"lse is null" in lib.distca_last_error()
+    assert fwd(q=None) == -1
+    assert need > 16
+    needb = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+    bwd = lambda **kw: lib.distca_ca_bwd_tokens(*[kw.get(n, d) for n, d in (
+        ("req", ptr), ("req_off", ptr), ("req_tok", 3 * row + 32), ("k", ptr), ("v", ptr), ("dq", ptr), ("dq_off", ptr), ("dq_tok", row),
+        ("dk", ptr), ("dv", ptr), ("cu_q", ptr), ("cu_k", ptr), ("kv_off", None), ("p", ctypes.byref(kw.get("params", p))), ("ws", ptr),
+        ("ws_bytes", 64), ("stream", None))])
+    assert bwd() == -3 and needb > 64
+    assert bwd(req_tok=3 * row) == -1 and b"request token" in lib.distca_last_error()
+    assert bwd(dq_tok=row - 16) == -1 and b"dq token" in lib.distca_last_error()
+    assert bwd(req_off=None) == -1 and b"offset" in lib.distca_last_error()
+    p6 = _lib.CaParams(2, 64, 64, 6, 2, 128, 32, 32, 0.088, 1, 0, 0)
+    assert bwd(params=p6) == -2 and b"alignment" in lib.distca_last_error()

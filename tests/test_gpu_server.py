@@ -233,9 +233,14 @@ def test_server_tick_from_single_rank_plan(cuda):
     fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
     gsend = torch.zeros(b_send, dtype=torch.uint8, device=cuda)
     print("plan backward", flush=True)
-    ca_server_backward(torch.from_numpy(recv).to(cuda), gsend, bmeta, fa_args, fa_params.cu_seqlens_q,
-                       fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
+    got = ca_server_backward(torch.from_numpy(recv).to(cuda), gsend, bmeta, fa_args, fa_params.cu_seqlens_q,
+                             fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
+    assert got[0] is None, "8 query heads: the kernels read the request and write dq in place"
+    gsend_steps = torch.zeros_like(gsend)
+    ca_server_backward(torch.from_numpy(recv).to(cuda), gsend_steps, bmeta, fa_args, fa_params.cu_seqlens_q,
+                       fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, in_place=False)
     torch.cuda.synchronize()
+    assert torch.equal(gsend, gsend_steps), "in-place and step-by-step ticks leave the same bytes"
     gq_off, gk_off, gv_off, _ = plan.reply_layout(True)
     g = gsend.cpu().numpy()
     dq = np.zeros((T, plan.q_bytes), np.uint8); dk = np.zeros((T, plan.k_bytes), np.uint8); dv = np.zeros_like(dk)
