@@ -39,6 +39,8 @@
 #include "attn_cfg.h"
 #include "common.h"
 
+#include <type_traits>
+
 namespace distca {
 namespace {
 
@@ -248,23 +250,31 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
     const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
     const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
+    // the masked form only for tiles that straddle the diagonal or the end of the task (uniform branch):
+    // compare and select per element are a third of this phase's instructions
+    auto body = [&](auto masked) __attribute__((always_inline)) {
 #pragma unroll
-    for (int cq = 0; cq < 4; ++cq) {
-      const int qr = 8 * cq + 4 * g;
-      const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
-      const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
-      i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
-      if (need_mask) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
+      for (int cq = 0; cq < 4; ++cq) {
+        const int qr = 8 * cq + 4 * g;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
+        i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+        if constexpr (decltype(masked)::value) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int r = 4 * cq + rr;
-        float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
-        if (need_mask && kw0 + l32 > lim4[rr]) p = 0.f;
-        const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
-        sacc[r] = p;
-        dpacc[r] = ds;
+        for (int rr = 0; rr < 4; ++rr) {
+          const int r = 4 * cq + rr;
+          float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
+          if constexpr (decltype(masked)::value) {
+            if (kw0 + l32 > lim4[rr]) p = 0.f;
+          }
+          const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
+          sacc[r] = p;
+          dpacc[r] = ds;
+        }
       }
-    }
+    };
+    if (need_mask) body(std::true_type{});
+    else body(std::false_type{});
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int r0 = 8 * t;
@@ -568,14 +578,21 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       bf16x8 dsf[MSUB][4];
 #pragma unroll
       for (int m = 0; m < MSUB; ++m) {
+        // the masked form only for tiles that straddle the diagonal or the end of the prefix (uniform branch)
+        auto body = [&](auto masked) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+          for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, -lse2[m]));
-            if (need_mask && key0 + kb * 32 + acc_row(r, g) > lim[m]) p = 0.f;
-            dpacc[m][kb][r] = p * __builtin_fmaf(dpacc[m][kb][r], a.scale, -dsc[m]);
-          }
+            for (int r = 0; r < 16; ++r) {
+              float p = fast_exp2(__builtin_fmaf(sacc[m][kb][r], c, -lse2[m]));
+              if constexpr (decltype(masked)::value) {
+                if (key0 + kb * 32 + acc_row(r, g) > lim[m]) p = 0.f;
+              }
+              dpacc[m][kb][r] = p * __builtin_fmaf(dpacc[m][kb][r], a.scale, -dsc[m]);
+            }
+        };
+        if (need_mask) body(std::true_type{});
+        else body(std::false_type{});
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const int kb = t >> 1, r0 = 8 * (t & 1);
