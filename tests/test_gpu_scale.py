@@ -282,3 +282,44 @@ def test_ops_replay_from_a_captured_graph(cuda):
         torch.cuda.synchronize()
         for name, a_, b_ in zip(("out", "lse", "dq", "dk", "dv", "buf"), got, (out, lse, dq, dk, dv, buf)):
             assert torch.equal(a_, b_), f"replay {rep}: {name} differs from the eager result"
+
+
+def test_server_ticks_in_place_equal_step_by_step_at_full_size(cuda):
+    """The 131072-token workload as one CA-server tick: the kernels that read request tokens from the
+    receive buffer and write reply tokens into the send buffer leave exactly the bytes the unpack ->
+    attention -> pack sequence leaves, forward and backward."""
+    from distca_amd import metadata, workloads
+    from distca_amd.fused_comm_attn import FlashAttnArgs, ca_server_backward, ca_server_forward
+    batch = workloads.config2_llama8b_128k()
+    plan = metadata.single_rank_plan([[int(n)] for n in batch.q_lens], 32, 8)
+    attn, fwd, bwd, (f_recv, f_send, b_recv, b_send) = metadata.server_metas(plan, cuda)
+    fa = FlashAttnArgs(32, 8, 128)
+    g = torch.Generator(device=cuda).manual_seed(3)
+    rnd_bytes = lambda n: torch.randn(n // 2, generator=g, device=cuda).to(torch.bfloat16).view(torch.uint8)
+    recv = rnd_bytes(f_recv)
+    sends = []
+    for in_place in (True, False):
+        send = torch.zeros(f_send, dtype=torch.uint8, device=cuda)
+        print(f"forward tick in_place={in_place}", flush=True)
+        ca_server_forward(recv, send, fwd, attn, fa, in_place=in_place)
+        sends.append(send)
+    torch.cuda.synchronize()
+    assert torch.equal(sends[0], sends[1])
+    # backward: any bytes will do as a request (the lse part is read as fp32: keep it finite and large
+    # enough that P stays below 1, as a real lse would)
+    breq = rnd_bytes(b_recv)
+    row = 32 * 128 * 2
+    tok = plan.merged_q_bytes
+    q_off = plan.request_layout(True)[0]
+    assert int(q_off[0]) == 0 and tok % 4 == 0
+    tokens = breq[:plan.num_q_tokens * tok].view(plan.num_q_tokens, tok)
+    tokens[:, 2 * row:2 * row + 32 * 4] = torch.full((plan.num_q_tokens, 32), 20.0, device=cuda).view(torch.uint8)
+    sends = []
+    for in_place in (True, False):
+        send = torch.zeros(b_send, dtype=torch.uint8, device=cuda)
+        print(f"backward tick in_place={in_place}", flush=True)
+        ca_server_backward(breq, send, bwd, fa, attn.cu_seqlens_q, attn.cu_seqlens_kv, attn.max_seqlen_q, attn.max_seqlen_kv,
+                           in_place=in_place)
+        sends.append(send)
+    torch.cuda.synchronize()
+    assert torch.equal(sends[0], sends[1])
