@@ -10,23 +10,24 @@
 // (row, key) pair per 128 keys, 124 GB at 128K tokens) took as long as the rest of the kernel.
 //
 //   1. bwd_prepare_kernel: per (token, head) row, scale*<dO, O> and lse*log2(e) -> workspace.
-//   2. ca_bwd_dkdv_kernel: one workgroup of 8 waves per (task, block of 128 keys, kv head),
+//   2. ca_bwd_dkdv_kernel: one workgroup of 8 waves per (task, block of 256 keys, kv head),
 //      in the order of the backward tile schedule.  V of the block sits in LDS for the
-//      workgroup's life, K in registers (each wave's 32 keys as B operand).  The query side (Q, dO and the two row statistics of every head of
-//      the kv group, flattened into rows like the forward) is streamed in blocks of 32 rows
-//      from the first block the causal mask lets see these keys.  The waves form two groups of
-//      four; per iteration group 0 takes query block 2i and group 1 block 2i+1, so that every
-//      SIMD holds two waves at different points of the loop body.  In a group wave w owns
-//      keys 32w..32w+31:
+//      workgroup's life, K in registers (each wave's 32 keys as B operand; the waves form two
+//      groups of four, group 0 with the block's first 128 keys, group 1 with the rest).  The
+//      query side (Q, dO and the two row statistics of every head of the kv group, flattened into
+//      rows like the forward) is streamed in blocks of 32 rows from the first block the causal
+//      mask lets see these keys; both groups work through every block, half a period apart, so
+//      that every SIMD holds two waves at different points of the loop body and a block is
+//      fetched once for 256 keys.  Per block and wave:
 //        S = Q K^T, dP = dO V^T            A from the query tile, B = K registers / V tile (LDS)
 //        P = exp2(S*c - lse2), dS = P (dP*scale - delta*scale)          in registers
 //        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
 //                                          B = the accumulator registers converted to bf16
-//      Query tiles arrive one iteration ahead through LDS-direct global loads, four 256-byte
-//      rows per instruction; the tile has unpadded rows whose 16-byte chunks are swizzled
-//      (tile_swz), which serves both read shapes without bank conflicts.  After the loop
-//      group 1 hands its partial sums to group 0 through LDS.
-//   3. ca_bwd_dq_kernel: one workgroup of 4 waves per (task, block of 128 flattened query
+//      Query tiles arrive two periods ahead through LDS-direct global loads (each wave brings
+//      four 256-byte rows of Q and of dO per tile, one instruction each) into a ring of four
+//      stages; the tile has unpadded rows whose 16-byte chunks are swizzled (tile_swz), which
+//      serves both read shapes without bank conflicts.
+//   3. ca_bwd_dq_kernel: one workgroup of 8 waves per (task, block of 256 flattened query
 //      rows, kv head), in the order of the forward tile schedule; the mirror image of the
 //      forward kernel.  Q and dO stay in registers as B operands, K/V tiles of 64 keys are
 //      streamed through LDS:
@@ -51,21 +52,22 @@ constexpr float kLog2e = 1.4426950408889634f;
 // dK / dV
 // ------------------------------------------------------------------------------------------
 constexpr int kBwdThreads = 512;
-constexpr int kBN = kBwdKV;    // 128 keys per workgroup
+constexpr int kBN = kBwdKV;    // 256 keys per workgroup
 constexpr int kBM = kBwdRows;  // 32 flattened query rows per block
 
-// LDS map (bytes)
-constexpr int kKsOff = 0;
-constexpr int kVsOff = kKsOff + kBN * kPitch;
-constexpr int kTileOff = kVsOff + kBN * kPitch;
+// LDS map (bytes): V of the block for the workgroup's life; behind it a region that first stages K on
+// its way into registers and then holds the ring of query-side tiles
+constexpr int kVsOff = 0;
+constexpr int kKsOff = kVsOff + kBN * kPitch;
+constexpr int kTileOff = kKsOff;
 constexpr int kTileRow = 256;                     // query-side tiles: unpadded rows, swizzled chunks (tile_swz)
 constexpr int kTileQ = 0, kTileDO = kBM * kTileRow;
 constexpr int kTileBytes = 2 * kBM * kTileRow;    // Q + dO of one block
-constexpr int kStatOff = kTileOff + 4 * kTileBytes;  // tiles: [stage 0/1][group 0/1]
-constexpr int kStatBytes = 3 * kBM * 4;           // per (stage, group): lse2, dscaled, lim
-constexpr int kBwdLds = kStatOff + 4 * kStatBytes;
-constexpr int kRedBytes = 4 * 64 * 64 * 4;        // group hand-over of one accumulator set
-static_assert(kRedBytes <= kTileOff, "reduction buffer must fit in the K/V region");
+constexpr int kStages = 4;                        // a tile is requested two periods ahead and read for a period and a half
+constexpr int kStatOff = kTileOff + kStages * kTileBytes;
+constexpr int kStatBytes = 3 * kBM * 4;           // per stage: lse2, dscaled, lim
+constexpr int kBwdLds = kKsOff + kBN * kPitch;
+static_assert(kStatOff + kStages * kStatBytes <= kBwdLds, "tile ring must fit in the K staging region");
 static_assert(kBwdLds <= 160 * 1024, "LDS budget");
 
 struct BwdArgs {
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   const int grp = wave >> 2, kbw = wave & 3;
   const int l32 = lane & 31, g = lane >> 5;
   const int kb0 = nblk * kBN;      // first key of the workgroup
-  const int kw0 = kb0 + kbw * 32;  // first key of the wave
+  const int kw0 = kb0 + (grp * 4 + kbw) * 32;  // first key of the wave: group 0 the block's first 128 keys, group 1 the rest
 
   int mb0 = 0;
   if (a.causal) {
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     if (t_first < 0) t_first = 0;
     mb0 = (int)(((int64_t)t_first * G) / kBM);
   }
-  const int niter = nmb > mb0 ? (nmb - mb0 + 1) / 2 : 0;
+  const int niter = nmb > mb0 ? nmb - mb0 : 0;
 
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
@@ -162,30 +164,29 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // The fetch of one block in three pieces: row statistics, rows 0-3, rows 4-7 of this wave's share.
   // (Issuing them between the MFMAs of phase A, as the forward kernel does, measured 2 % slower here:
   // the other group is in its LDS-bound phase C at that time.)
-  auto issue_piece = [&](int stage, int mbx, int piece) {
-    const int tile = kTileOff + (stage * 2 + grp) * kTileBytes;
-    const int stat = kStatOff + (stage * 2 + grp) * kStatBytes;
+  auto issue_tile = [&](int stage, int mbx) {
+    const int tile = kTileOff + stage * kTileBytes;
+    const int stat = kStatOff + stage * kStatBytes;
     const bool blk_ok = mbx >= mb0;
-    if (piece == 0) {  // row statistics: lanes 0..7 take one row each
-      const int rl = kbw * 8 + (lane & 7);
+    {  // row statistics: lanes 0..3 take one of the wave's four rows each
+      const int rl = wave * 4 + (lane & 3);
       const int rho = mbx * kBM + rl;
       const bool ok = blk_ok && rho < nrows;
       const int rc = ok ? rho : nrows - 1;
       const int tok = div_group(rc);
       const int hg = rc - tok * G;
-      if (lane < 8) {
+      if (lane < 4) {
         int lm = a.causal ? tok + shift : lk - 1;
         if (lm > lk - 1) lm = lk - 1;
         reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
         const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
-        lds_direct_load4(a.lse2 + so, lds0 + stat + kbw * 32);
-        lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + kbw * 32);
+        lds_direct_load4(a.lse2 + so, lds0 + stat + wave * 16);
+        lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + wave * 16);
       }
-    } else {
-      // Q and dO: one instruction fills four rows; lane p brings the chunk that belongs at chunk
-      // position p%16 of row p/16.  Rows that do not exist read the zero row.
-      const int i = piece - 1;
-      const int rl = kbw * 8 + 4 * i + (lane >> 4);
+    }
+    {  // Q and dO: one instruction fills the wave's four rows; lane p brings the chunk that belongs at
+       // chunk position p%16 of row p/16.  Rows that do not exist read the zero row.
+      const int rl = wave * 4 + (lane >> 4);
       const int rho = mbx * kBM + rl;
       const bool ok = blk_ok && rho < nrows;
       const int tok = div_group(ok ? rho : 0);
@@ -194,20 +195,18 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       const int64_t eo = qbase + (int64_t)tok * a.qs_tok_bytes + hg * (kHeadDim * 2);
       const __bf16 *qs = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
       const __bf16 *ds = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
-      const uint32_t dst = lds0 + tile + (kbw * 8 + 4 * i) * kTileRow;
+      const uint32_t dst = lds0 + tile + wave * 4 * kTileRow;
       lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
       lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
     }
   };
-  auto issue_tile = [&](int stage, int mbx) {
-#pragma unroll
-    for (int piece = 0; piece < 3; ++piece) issue_piece(stage, mbx, piece);
-  };
+  // a wave has four fetch instructions per tile; older tiles have landed once at most that many are pending
+  auto wait_older = [&]() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); };
 
   const float c = a.scale * kLog2e;
   // tile-independent LDS offsets
   const int a_rd = l32 * kTileRow + ((g ^ tile_swz(l32)) << 4);  // A operand rows of the query tile, ^ 32*s
-  const int b_rd = (kbw * 32 + l32) * kPitch + 16 * g;           // B operand rows of K / V, + 32*s
+  const int b_rd = ((grp * 4 + kbw) * 32 + l32) * kPitch + 16 * g;  // B operand rows of K / V, + 32*s
   // transposed A operand: lane points at (row 4g + i4 [+8 hi +16 (j>>2)], chunk 8 b4 + h1 [+2 (j&3)], half lane&1);
   // tile_swz of that row is (i4<<1) | (g<<3) | hi
   const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
@@ -217,7 +216,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   f32x16 sacc, dpacc;
   // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
   auto phase_a = [&](int stage) {
-    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+    const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       sacc[r] = 0.f;
@@ -246,7 +245,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // ---- phase B (VALU): P and dS, converted to bf16 B operands
   bf16x8 pb[2], dsb[2];
   auto phase_b = [&](int stage) {
-    const uint8_t *stat = lds + kStatOff + (stage * 2 + grp) * kStatBytes;
+    const uint8_t *stat = lds + kStatOff + stage * kStatBytes;
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
     const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
     const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
@@ -284,7 +283,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   };
   // ---- phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
   auto phase_c = [&](int stage) {
-    const uint8_t *tile = lds + kTileOff + (stage * 2 + grp) * kTileBytes;
+    const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
     constexpr int kDc = 2;  // operand fetch distance in MFMA steps
     bf16x4 ct[kDc][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
     auto load_c = [&](int j, int buf) {
@@ -307,79 +306,60 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     }
   };
 
-  // The two groups run half a period apart: between the first and the second barrier of a
-  // period group 0 is in its MFMA-only phase A while group 1 starts with the VALU-heavy
-  // phase B; after the second barrier the roles swap.  A SIMD holds one wave of each
-  // group, so its MFMA pipe and its VALU are busy at the same time instead of by turns.
-  //   period p:  [barrier 1]  g0: fetch(p+1), A(p)   g1: B,C(p-1)
-  //              [barrier 2]  g0: B,C(p)             g1: fetch(p+1), A(p)
-  // (Moving B in front of the second barrier, which evens out the instruction counts of the two
-  // halves, measured 14 % slower: phases A and C both live on LDS reads and then run together.)
-  // A group's tile p+1 is requested right after the barrier that retires tile p-1 and is
-  // waited for before the same barrier one period later.
-  // Each group has its own copy of the loop (every wave still passes the same 2*(niter+1)
-  // barriers), which keeps the register allocation of either path as small as a single loop's.
+  // Both groups work through every tile, half a period apart: between barriers b1(p) and b2(p) group 0
+  // is in its MFMA-only phase A of tile p while group 1 does the arithmetic phase B and then phase C of
+  // tile p-1; after b2(p) the roles swap.  A SIMD holds one wave of each group, so its MFMA pipe and its
+  // VALU are busy at the same time instead of by turns.
+  //   [b1(p), b2(p)):    g0: fetch(p+2), A(p)     g1: B(p-1), C(p-1)
+  //   [b2(p), b1(p+1)):  g0: B(p), C(p)           g1: fetch(p+2), A(p)
+  // (Moving B in front of b2, which evens out the instruction counts of the two halves, measured 14 %
+  // slower: phases A and C both live on LDS reads and then run together.)
+  // Tile p is read from b1(p) to b2(p+1).  Every wave requests its four rows of tile p+2 at the start of
+  // its phase A of tile p, into the stage tile p-2 left at b2(p-1), and makes sure before each b1 that at
+  // most its newest request is pending, so that tile p is complete at b1(p).  Requests are made for
+  // tiles past the end as well (their rows come from the zero row), which keeps that count fixed.
+  // Each group has its own copy of the loop (every wave passes the same 2*niter + 1 barriers), which
+  // keeps the register allocation of either path as small as a single loop's.
   // Blocks are visited from the last one down to the diagonal: workgroups that run at the
   // same time (neighbouring key blocks of one document, by the schedule) then read the same
   // query rows at the same time and find them in their XCD's L2.
-  if (niter > 0) issue_tile(0, nmb - 1 - grp);
   __syncthreads();
 #pragma unroll
   for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
+  __syncthreads();  // K has left LDS: its region now holds the tile ring
+  if (niter > 0) {
+    issue_tile(0, nmb - 1);
+    issue_tile(1, nmb - 2);
+  }
+  wait_vm0();
   if (grp == 0) {
     for (int p = 0; p < niter; ++p) {
-      const int stage = p & 1;
-      wait_vm0();
-      __syncthreads();
-      if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 1 - 2 * (p + 1));
-      phase_a(stage);
-      __syncthreads();
-      phase_b(stage);
-      phase_c(stage);
+      wait_older();
+      __syncthreads();  // b1(p): tile p is complete
+      issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      phase_a(p % kStages);
+      __syncthreads();  // b2(p)
+      phase_b(p % kStages);
+      phase_c(p % kStages);
     }
-    __syncthreads();
-    __syncthreads();
+    __syncthreads();  // b1(niter), which group 1 passes between its last phases A and B
   } else {
-    __syncthreads();
+    __syncthreads();    // b1(0)
     for (int p = 0; p < niter; ++p) {
-      const int stage = p & 1;
-      wait_vm0();
-      __syncthreads();
-      if (p + 1 < niter) issue_tile(stage ^ 1, nmb - 2 - 2 * (p + 1));
-      phase_a(stage);
-      __syncthreads();
-      phase_b(stage);
-      phase_c(stage);
-    }
-    __syncthreads();
-  }
-
-  // ---- group 1 hands its partial dK^T / dV^T to group 0 through LDS (K/V region, no longer read)
-  float *red = reinterpret_cast<float *>(lds) + (kbw * 64) * 64 + lane;
-#pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    __syncthreads();
-    if (grp == 1) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) red[(db * 16 + r) * 64] = pass == 0 ? dkacc[db][r] : dvacc[db][r];
-    }
-    __syncthreads();
-    if (grp == 0) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          if (pass == 0) dkacc[db][r] += red[(db * 16 + r) * 64];
-          else dvacc[db][r] += red[(db * 16 + r) * 64];
-        }
+      __syncthreads();  // b2(p)
+      issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      phase_a(p % kStages);
+      wait_older();
+      __syncthreads();  // b1(p+1): tile p+1 is complete
+      phase_b(p % kStages);
+      phase_c(p % kStages);
     }
   }
+  wait_vm0();  // nothing may still be on its way into LDS when the workgroup ends
 
   // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
   const int key = kw0 + l32;
-  if (grp == 0 && key < lk) {
+  if (key < lk) {
     const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -855,7 +835,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve LDS");
   }
 
-  // ---- dK, dV: one workgroup per (task, 128-key block, kv head)
+  // ---- dK, dV: one workgroup per (task, 256-key block, kv head)
   {
     const SchedGeom geom = bwd_geom(p);
     const int64_t max_items = bwd_max_items(p);

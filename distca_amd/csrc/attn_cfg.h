@@ -28,10 +28,10 @@ constexpr int kFwdRows = kFwdWaves * 32 * kFwdMsub;
 constexpr int kDqRows = kWaves * 32 * kFwdMsub;
 constexpr int kFwdKV = 64;
 
-// Backward: a workgroup owns 128 keys (four waves of 32, in two copies that take alternate
-// query blocks); query rows are streamed in blocks of 32 flattened rows.
+// Backward: a workgroup owns 256 keys (eight waves of 32, in two groups that work through the same
+// query blocks half a period apart); query rows are streamed in blocks of 32 flattened rows.
 constexpr int kBwdRows = 32;
-constexpr int kBwdKV = 128;
+constexpr int kBwdKV = 256;
 
 inline int validate_params(const distca_ca_params *p) {
   if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: this build has kernels for head_dim 128 only", p->head_dim);
