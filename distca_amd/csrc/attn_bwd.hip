@@ -758,7 +758,8 @@ extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_tas
   const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2, lse_bytes = (int64_t)p->num_heads_q * 4;
   if (lse_bytes & 15)
     return fail(DISTCA_E_UNSUPPORTED, "ca_bwd_tokens: %d query heads put the q part of a request token off 16-byte alignment", p->num_heads_q);
-  if (!req_task_off || !dq_task_off) return fail(DISTCA_E_INVALID, "ca_bwd_tokens: null offset array");
+  // a server with no task this tick has empty offset arrays, which may come as null pointers; nothing reads them then
+  if ((!req_task_off || !dq_task_off) && p->num_tasks > 0) return fail(DISTCA_E_INVALID, "ca_bwd_tokens: null offset array");
   if (req_tok_bytes < 3 * row_bytes + lse_bytes || (req_tok_bytes & 15))
     return fail(DISTCA_E_INVALID, "ca_bwd_tokens: request token of %lld B (needs >= %lld, multiple of 16)", (long long)req_tok_bytes, (long long)(3 * row_bytes + lse_bytes));
   if (dq_tok_bytes < row_bytes || (dq_tok_bytes & 15))

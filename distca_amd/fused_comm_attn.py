@@ -9,6 +9,7 @@ there is no other attention implementation behind these functions.
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 from dataclasses import dataclass
 from typing import Optional, Tuple
@@ -431,7 +432,7 @@ def post_a2a_attn_out_with_lse(recv_buffer: Tensor, q: Tensor, num_heads_q: int,
     recv = torch.empty(recv_shape, dtype=dtype, device=recv_buffer.device).view(torch.uint8)
     post_a2a_attn_out(recv, metadata.seq_lens[0].recv_seqlens, *metadata.recv_memcpy_metadata, buffer=recv_buffer)
     itemsize = torch.empty((), dtype=dtype).element_size()
-    hidden_bytes = int(q.numel() // q.shape[0]) * itemsize
+    hidden_bytes = math.prod(q.shape[1:]) * itemsize
     lse_bytes = num_heads_q * 4
     attn_out = recv[:, :hidden_bytes].contiguous().view(dtype).unsqueeze(1)
     softmax_lse_bytes = recv[:, hidden_bytes:hidden_bytes + lse_bytes]
@@ -442,7 +443,7 @@ def post_a2a_attn_out_with_lse_backward(send_buffer: Tensor, grad_attn_out: Tens
                                         q: Tensor, k: Tensor, v: Tensor, bwd_attn_out_qkv_metadata):
     """Linear side, backward of the same function (fused_comm_attn.py:508-526): pack the request
     [dO | O | lse | q | pad] and the K/V shards for the attention server."""
-    flat = lambda t: t.reshape(t.shape[0], -1)
+    flat = lambda t: t.reshape(t.shape[0], math.prod(t.shape[1:]))   # -1 is ambiguous for a rank that holds no tokens
     md = bwd_attn_out_qkv_metadata
     pre_a2a_attn_out_grad_resend_qkv(
         flat(grad_attn_out), flat(attn_out), softmax_lse_bytes, flat(q), flat(k), flat(v), md.kv_replica_mask,

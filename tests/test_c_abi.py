@@ -197,3 +197,11 @@ def test_token_layout_entry_points_check_their_layouts():
     assert bwd(req_off=None) == -1 and b"offset" in lib.distca_last_error()
     p6 = _lib.CaParams(2, 64, 64, 6, 2, 128, 32, 32, 0.088, 1, 0, 0)
     assert bwd(params=p6) == -2 and b"alignment" in lib.distca_last_error()
+    # a server without a task this tick: empty (null) arrays everywhere, nothing to do, no error
+    idle = _lib.CaParams(0, 0, 0, 8, 2, 128, 0, 0, 0.088, 1, 0, 0)
+    nothing = dict(req=None, req_off=None, k=None, v=None, dq=None, dq_off=None, dk=None, dv=None, cu_q=None, cu_k=None, ws=None, ws_bytes=0)
+    assert bwd(params=idle, **nothing) == 0
+    p_save = p
+    p = idle
+    assert fwd(q=None, q_off=None, k=None, v=None, out=None, out_off=None, cu_q=None, cu_k=None, ws=None, ws_bytes=0) == 0
+    p = p_save
