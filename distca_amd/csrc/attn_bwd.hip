@@ -77,6 +77,7 @@ struct BwdArgs {
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;
+  int32_t *tickets;  // one counter per kv head (sched.h)
   const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
   int32_t sched_items_off;
   int32_t hq, hkv, group, total_q;
@@ -94,9 +95,8 @@ template <bool ALIAS>
 __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
-  const int item = blockIdx.x / a.hkv;
-  if (item >= nitems) return;
-  const int kvh = blockIdx.x - item * a.hkv;
+  int item, kvh;
+  if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
   const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
   const int task = it4.x, nblk = it4.y;
 
@@ -270,6 +270,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
           sacc[r] = p;
           dpacc[r] = ds;
         }
+        if (cq == 1) __builtin_amdgcn_sched_barrier(0);  // at most half of the row statistics in registers at a time
       }
     };
     if (need_mask) body(std::true_type{});
@@ -318,6 +319,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // its phase A of tile p, into the stage tile p-2 left at b2(p-1), and makes sure before each b1 that at
   // most its newest request is pending, so that tile p is complete at b1(p).  Requests are made for
   // tiles past the end as well (their rows come from the zero row), which keeps that count fixed.
+  // A wave raises its priority for its MFMA phases: the instruction arbiter prefers the older wave
+  // of a SIMD, which otherwise lets group 0's arithmetic phase hold up group 1's MFMAs (-1.3 %).
   // Each group has its own copy of the loop (every wave passes the same 2*niter + 1 barriers), which
   // keeps the register allocation of either path as small as a single loop's.
   // Blocks are visited from the last one down to the diagonal: workgroups that run at the
@@ -337,10 +340,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       wait_older();
       __syncthreads();  // b1(p): tile p is complete
       issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      __builtin_amdgcn_s_setprio(3);
       phase_a(p % kStages);
+      __builtin_amdgcn_s_setprio(0);
       __syncthreads();  // b2(p)
       phase_b(p % kStages);
+      __builtin_amdgcn_s_setprio(3);
       phase_c(p % kStages);
+      __builtin_amdgcn_s_setprio(0);
     }
     __syncthreads();  // b1(niter), which group 1 passes between its last phases A and B
   } else {
@@ -348,11 +355,15 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     for (int p = 0; p < niter; ++p) {
       __syncthreads();  // b2(p)
       issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      __builtin_amdgcn_s_setprio(3);
       phase_a(p % kStages);
+      __builtin_amdgcn_s_setprio(0);
       wait_older();
       __syncthreads();  // b1(p+1): tile p+1 is complete
       phase_b(p % kStages);
+      __builtin_amdgcn_s_setprio(3);
       phase_c(p % kStages);
+      __builtin_amdgcn_s_setprio(0);
     }
   }
   wait_vm0();  // nothing may still be on its way into LDS when the workgroup ends
@@ -395,9 +406,8 @@ template <int MSUB>
 __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) void ca_bwd_dq_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
-  const int item = blockIdx.x / a.hkv;
-  if (item >= nitems) return;
-  const int kvh = blockIdx.x - item * a.hkv;
+  int item, kvh;
+  if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
   const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
   const int task = it4.x, mblk = it4.y;
 
@@ -842,10 +852,11 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     const int64_t max_items = bwd_max_items(p);
     rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_kv), max_items, s);
     if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv;
+    const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_kv);
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
+    a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     if (alias)
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
@@ -858,10 +869,11 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     const int64_t max_items = dq_max_items(p);
     rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
     if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv;
+    const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_q);
     a.zero_row = ws + w.sched_q + sched_zero_row_off(p->num_tasks, max_items);
+    a.tickets = (int32_t *)(ws + w.sched_q + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
     hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
   }

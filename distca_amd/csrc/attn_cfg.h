@@ -37,6 +37,7 @@ inline int validate_params(const distca_ca_params *p) {
   if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: this build has kernels for head_dim 128 only", p->head_dim);
   if (p->num_heads_q <= 0 || p->num_heads_kv <= 0 || p->num_heads_q % p->num_heads_kv)
     return fail(DISTCA_E_INVALID, "num_heads_q=%d must be a positive multiple of num_heads_kv=%d", p->num_heads_q, p->num_heads_kv);
+  if (p->num_heads_kv > kSchedMaxHeads) return fail(DISTCA_E_UNSUPPORTED, "num_heads_kv=%d: at most %d kv heads", p->num_heads_kv, kSchedMaxHeads);
   if (p->num_tasks < 0 || p->total_q < 0 || p->total_k < 0 || p->max_seqlen_q < 0 || p->max_seqlen_k < 0)
     return fail(DISTCA_E_INVALID, "negative size in distca_ca_params");
   if (!(p->softmax_scale > 0.f) || !isfinite(p->softmax_scale)) return fail(DISTCA_E_INVALID, "softmax_scale must be positive and finite");

@@ -50,6 +50,7 @@ struct FwdArgs {
   float scale;
   // Where the query and output tokens live.  Token t of task b starts at base + off[b] + t * tok_bytes
   // (off == nullptr: the packed tensor, off[b] = cu_q[b] * tok_bytes); head h at + h * 256 bytes.
+  int32_t *tickets;  // one counter per kv head (sched.h)
   const int64_t *q_task_off, *out_task_off;
   int64_t q_tok_bytes, out_tok_bytes;
   int32_t lse_in_token;  // 1: lse of (token, head) as fp32 at token + hq * 256 + h * 4 (the [out | lse] reply), 0: lse[h][token]
@@ -59,9 +60,8 @@ template <int MSUB>
 __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
-  const int item = blockIdx.x / a.hkv;
-  if (item >= nitems) return;
-  const int kvh = blockIdx.x - item * a.hkv;
+  int item, kvh;
+  if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
   const int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
   const int task = it.x, mblk = it.y;
 
@@ -429,11 +429,12 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   a.sched = (const int32_t *)workspace;
   a.zero_row = (const uint8_t *)workspace + sched_zero_row_off(p->num_tasks, max_items);
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
+  a.tickets = (int32_t *)((uint8_t *)workspace + sched_ticket_off(p->num_tasks, max_items));
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   a.q_task_off = q_task_off; a.out_task_off = out_task_off; a.q_tok_bytes = q_tok_bytes; a.out_tok_bytes = out_tok_bytes;
   a.lse_in_token = lse ? 0 : 1;
-  const int64_t grid = max_items * p->num_heads_kv;
+  const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
   if (first_use_on_this_device(kSlotFwdLds)) {
     hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);

@@ -1,10 +1,10 @@
 // Tile scheduler: turns (cu_seqlens_q, cu_seqlens_k) into a list of work items sorted by
-// descending cost.  The attention kernels are launched with one workgroup per
-// (item, kv-head) in list order, workgroup id = item_rank * Hkv + kv_head.  The hardware
-// dispatcher hands workgroups to compute units in id order as slots free up, so a sorted
-// list gives longest-processing-time-first balancing across CUs without a persistent
-// kernel or atomics; and because workgroup ids are dealt round-robin over the 8 XCDs,
-// with Hkv = 8 every XCD works on one kv head and its L2 holds only that head's K/V.
+// descending cost, from which the attention kernels' workgroups draw: every workgroup takes
+// the next item of its home kv head (workgroup id % Hkv), so that a compute unit that frees up
+// continues with the most expensive item left -- longest-processing-time-first balancing
+// without a persistent kernel.  Workgroup ids are dealt round-robin over the 8 XCDs, so with
+// Hkv = 8 every XCD works on one kv head and its L2 holds only that head's K/V, until that
+// head's list is used up (see the ticket counters below).
 //
 // Cost unit = the causal-pair count the reference's planner balances across ranks
 // (Item.get_flops, distca/planner/planner.py:366-378), here at tile granularity.
@@ -89,8 +89,48 @@ constexpr int64_t kZeroRowBytes = 256;
 DISTCA_HD int64_t sched_zero_row_off(int32_t num_tasks, int64_t max_items) {
   return (sched_bytes(num_tasks, max_items) + 255) / 256 * 256;
 }
-DISTCA_HD int64_t sched_region_bytes(int32_t num_tasks, int64_t max_items) {
+// After the zero row: one ticket counter per kv head, zeroed by the builder.  The attention kernels
+// are launched with kSchedOversub workgroups per (item, kv head).  A workgroup does not work on the
+// item its id names: it draws the next ticket of its home head (id % Hkv), which is the rank of its
+// item in the sorted list, and when that head's list is used up it draws from the other heads; it
+// exits when all are used up.  Workgroup ids are dealt round-robin over the XCDs, and the XCDs of one
+// device do not run at the same speed (several per cent apart on the same work): with one workgroup
+// per item the kernel lasted as long as the slowest XCD took for its fixed eighth of the list,
+// whereas now an XCD that finishes its own heads early takes items of the others.
+constexpr int64_t kTicketBytes = 1024;
+constexpr int32_t kSchedMaxHeads = (int32_t)(kTicketBytes / 4);
+constexpr int32_t kSchedOversub = 2;
+DISTCA_HD int64_t sched_ticket_off(int32_t num_tasks, int64_t max_items) {
   return sched_zero_row_off(num_tasks, max_items) + kZeroRowBytes;
 }
+DISTCA_HD int64_t sched_region_bytes(int32_t num_tasks, int64_t max_items) {
+  return sched_ticket_off(num_tasks, max_items) + kTicketBytes;
+}
+
+#if defined(__HIPCC__)
+// Draws this workgroup's (item rank, kv head); false when every list is used up.  `slot` is two ints
+// of LDS that the caller may reuse afterwards.  All threads of the workgroup must call it.
+__device__ __forceinline__ bool take_item(int32_t *tickets, int32_t nitems, int32_t hkv, int32_t *slot, int &item, int &kvh) {
+  if (threadIdx.x == 0) {
+    int q = (int)(blockIdx.x % (unsigned)hkv), t = -1;
+    for (int d = 0; d < hkv; ++d) {
+      // counters only grow: a list seen as used up stays so, and a stale smaller value only costs the atomic
+      if (__builtin_nontemporal_load(tickets + q) < nitems) {
+        t = atomicAdd(tickets + q, 1);
+        if (t < nitems) break;
+        t = -1;
+      }
+      if (++q == hkv) q = 0;
+    }
+    slot[0] = t;
+    slot[1] = q;
+  }
+  __syncthreads();
+  item = __builtin_amdgcn_readfirstlane(slot[0]);
+  kvh = __builtin_amdgcn_readfirstlane(slot[1]);
+  __syncthreads();
+  return item >= 0;
+}
+#endif
 
 }  // namespace distca

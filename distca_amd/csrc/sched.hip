@@ -119,6 +119,7 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
     ws[1] = running;
   }
   if (tid < kZeroRowBytes / 4) ws[sched_zero_row_off(num_tasks, max_items) / 4 + tid] = 0;
+  if (tid < kTicketBytes / 4) ws[sched_ticket_off(num_tasks, max_items) / 4 + tid] = 0;
 }
 
 }  // namespace
