@@ -164,10 +164,43 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // The fetch of one block in three pieces: row statistics, rows 0-3, rows 4-7 of this wave's share.
   // (Issuing them between the MFMAs of phase A, as the forward kernel does, measured 2 % slower here:
   // the other group is in its LDS-bound phase C at that time.)
+  // Blocks whose 32 rows all exist take a form without per-lane address arithmetic when the group size
+  // divides 32 (a block then starts at a token boundary): scalar bases that move by one block, plus per-lane
+  // offsets that never change.
+  const bool fast_ok = (kBM % G) == 0 && (int64_t)G * a.total_q * 4 < (1ll << 32) && 32 * a.qs_tok_bytes < (1ll << 32);
+  const int tok_per_blk = kBM / G;
+  uint32_t voff_q, voff_s;
+  int tok_s;
+  {
+    const int rl = wave * 4 + (lane >> 4);
+    const int tq = div_group(rl);
+    voff_q = (uint32_t)(tq * a.qs_tok_bytes + (rl - tq * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(rl)) << 4));
+    const int rs = wave * 4 + (lane & 3);
+    tok_s = div_group(rs);
+    voff_s = (uint32_t)((((int64_t)(rs - tok_s * G)) * a.total_q + tok_s) * 4);
+  }
+  const float *stat_base = a.lse2 + (int64_t)kvh * G * a.total_q + q0;
+  const int64_t stat_delta = a.dscaled - a.lse2;
   auto issue_tile = [&](int stage, int mbx) {
     const int tile = kTileOff + stage * kTileBytes;
     const int stat = kStatOff + stage * kStatBytes;
     const bool blk_ok = mbx >= mb0;
+    if (fast_ok && blk_ok && (mbx + 1) * kBM <= nrows) {
+      const int tok0 = mbx * tok_per_blk;
+      if (lane < 4) {
+        int lm = a.causal ? tok0 + tok_s + shift : lk - 1;
+        if (lm > lk - 1) lm = lk - 1;
+        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[wave * 4 + lane] = lm;
+        lds_direct_load4_base(stat_base + tok0, voff_s, lds0 + stat + wave * 16);
+        lds_direct_load4_base(stat_base + stat_delta + tok0, voff_s, lds0 + stat + kBM * 4 + wave * 16);
+      }
+      const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
+      const uint8_t *db = reinterpret_cast<const uint8_t *>(a.dout) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
+      const uint32_t dst = lds0 + tile + wave * 4 * kTileRow;
+      lds_direct_load16(qb, voff_q, dst + kTileQ);
+      lds_direct_load16(db, voff_q, dst + kTileDO);
+      return;
+    }
     {  // row statistics: lanes 0..3 take one of the wave's four rows each
       const int rl = wave * 4 + (lane & 3);
       const int rho = mbx * kBM + rl;
@@ -495,6 +528,20 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     const uint32_t dst = lds0 + stage * kDqStage + (is_k ? 0 : kDqTile) + (kRowsW * uwave + 4 * ii) * kDqRowB;
     lds_direct_load16_ptr(src + chunk * 8, dst);
   };
+  // Tiles that lie wholly inside the prefix (all but the last one) take a form without per-lane address
+  // arithmetic: a scalar base that advances by one tile, plus a per-lane offset that never changes.
+  uint32_t voff[kLdW / 2];
+#pragma unroll
+  for (int ii = 0; ii < kLdW / 2; ++ii) {
+    const int r = kRowsW * uwave + 4 * ii + (lane >> 4);
+    voff[ii] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
+  }
+  auto issue_kv_whole = [&](int j, int stage, int i) {
+    const bool is_k = i < kLdW / 2;
+    const int ii = is_k ? i : i - kLdW / 2;
+    const __bf16 *tb = (is_k ? kbase : vbase) + (int64_t)j * kDqKV * kv_stride;
+    lds_direct_load16(tb, voff[ii], lds0 + stage * kDqStage + (is_k ? 0 : kDqTile) + (kRowsW * uwave + 4 * ii) * kDqRowB);
+  };
 
   f32x16 dqacc[MSUB][4];
 #pragma unroll
@@ -524,6 +571,13 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
 
     const int key0 = j * kDqKV;
     const bool active = wave_live && key0 <= lim_last;
+    // the next tile: whole tiles are requested one instruction per MFMA step below; the one the end of the
+    // prefix cuts off (the last) needs per-lane addresses and is requested here
+    const bool next_whole = has_next && (j + 2) * kDqKV <= lk;
+    if (has_next && (!next_whole || !active)) {
+#pragma unroll
+      for (int i = 0; i < kLdW; ++i) issue_kv(j + 1, stage ^ 1, i);
+    }
     if (active) {
       // ---- S^T = K Q^T, dP^T = V dO^T : [64 keys] x [32*MSUB rows]
       f32x16 sacc[MSUB][2], dpacc[MSUB][2];
@@ -561,7 +615,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
           }
         __builtin_amdgcn_sched_barrier(0);
         if (s + kPf < 8) load_kv(s + kPf, s % kPf);
-        if (has_next && s < kLdW) issue_kv(j + 1, stage ^ 1, s);
+        if (next_whole && s < kLdW) issue_kv_whole(j + 1, stage ^ 1, s);
       }
       // ---- P, dS (one query row per lane) and the bf16 B operand of the dQ product
       const bool need_mask = key0 + kDqKV - 1 > lim_first;
@@ -608,10 +662,6 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
         __builtin_amdgcn_sched_barrier(0);
         if (u + kPfT < 16) load_t(u + kPfT, u % kPfT);
       }
-    } else if (has_next) {
-      // nothing to compute in this tile: still fetch this wave's share of the next one
-#pragma unroll
-      for (int i = 0; i < kLdW; ++i) issue_kv(j + 1, stage ^ 1, i);
     }
     wait_vm0();
     __syncthreads();

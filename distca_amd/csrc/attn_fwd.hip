@@ -147,8 +147,27 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
       lds_direct_load16_ptr(src + chunk * 8, lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
     }
   };
-  auto issue_k = [&](int j) { issue_rows(kbase, j, kKOff + (j & 1) * kKTile); };
-  auto issue_v = [&](int j) { issue_rows(vbase, j, kVOff + (j & 1) * kVTile); };
+  // Tiles that lie wholly inside the prefix (all but the last one) take a form without per-lane address
+  // arithmetic: a scalar base that advances by one tile, plus a per-lane offset that never changes.
+  uint32_t voff[kLdW];
+#pragma unroll
+  for (int i = 0; i < kLdW; ++i) {
+    const int r = kRowsW * uwave + 4 * i + (lane >> 4);
+    voff[i] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
+  }
+  auto issue_rows_fast = [&](const __bf16 *base, int j, uint32_t tile_off) {
+    const __bf16 *tb = base + (int64_t)j * kFwdKV * kv_stride;
+#pragma unroll
+    for (int i = 0; i < kLdW; ++i) lds_direct_load16(tb, voff[i], lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
+  };
+  auto issue_k = [&](int j) {
+    if ((j + 1) * kFwdKV <= lk) issue_rows_fast(kbase, j, kKOff + (j & 1) * kKTile);
+    else issue_rows(kbase, j, kKOff + (j & 1) * kKTile);
+  };
+  auto issue_v = [&](int j) {
+    if ((j + 1) * kFwdKV <= lk) issue_rows_fast(vbase, j, kVOff + (j & 1) * kVTile);
+    else issue_rows(vbase, j, kVOff + (j & 1) * kVTile);
+  };
 
   // ---- accumulators
   f32x16 oacc[MSUB][4];

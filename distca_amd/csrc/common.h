@@ -72,6 +72,11 @@ __device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t vo
 __device__ __forceinline__ void lds_direct_load16_ptr(const void *gptr_lane, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
 }
+__device__ __forceinline__ void lds_direct_load4_base(const void *gbase, uint32_t voff, uint32_t lds_base) {
+  const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
+  const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(gbu), "s"(uniform32(lds_base)) : "memory");
+}
 __device__ __forceinline__ void lds_direct_load4(const void *gptr_lane, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr_lane), "s"(uniform32(lds_base)) : "memory");
 }
