@@ -317,20 +317,23 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   //   [b(2p),   b(2p+1)):  group 0: PV(p-1), S(p)     group 1: softmax(p-1)
   //   [b(2p+1), b(2p+2)):  group 0: softmax(p)        group 1: PV(p-1), S(p)
   // Tile p of K is read between b(2p) and b(2p+2), tile p of V between b(2p+2) and b(2p+4); every
-  // wave requests K(p+1) and V(p) right after b(2p), into the stages whose last readers finished
-  // before that barrier, and waits for its own requests before b(2p+2).
+  // wave requests K(p+1) and V(p) at the start of its softmax half of period p (group 1 right after
+  // b(2p), group 0 right after b(2p+1)), into the stages whose last readers finished before b(2p), and
+  // waits for its own requests before b(2p+2).  The MFMA halves are the critical path of a period (one
+  // group's, then the other's); a request holds its wave for a hundred cycles or so, and in front of
+  // group 0's MFMA half that time showed in the period (-3 % with the requests behind it).
   const int grp = uwave >> 2;
   if (ntiles > 0) issue_k(0);
   wait_vm0();
   __syncthreads();  // b0
   if (grp == 0) {
     for (int p = 0; p <= ntiles; ++p) {
-      if (p + 1 < ntiles) issue_k(p + 1);
-      if (p < ntiles) issue_v(p);
       if (p > 0 && tile_active(p - 1)) phase_pv(p - 1);
       const bool act = p < ntiles && tile_active(p);
       if (act) phase_s(p);
       __syncthreads();
+      if (p + 1 < ntiles) issue_k(p + 1);
+      if (p < ntiles) issue_v(p);
       if (act) phase_x(p);
       wait_vm0();
       __syncthreads();
