@@ -563,10 +563,18 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   wait_vm0();
   __syncthreads();
 
-  for (int j = 0; j < ntiles; ++j) {
-    const int stage = j & 1;
-    const uint8_t *kt = lds + stage * kDqStage;
-    const uint8_t *vt = kt + kDqTile;
+  // Absolute LDS addresses of this lane's operand reads in stage 0, the eight swizzled variants of each, kept
+  // in registers; the tile loop is unrolled by two so that the stage is a constant in the instruction's offset
+  // field: no address arithmetic is left between the MFMAs.
+  uint32_t k_ad[8], t_ad[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    k_ad[i] = lds0 + (k_rd ^ (i << 5));
+    t_ad[i] = lds0 + (t_rd ^ ((i & 3) << 5) ^ ((i >> 2) << 4));
+    asm volatile("" : "+v"(k_ad[i]), "+v"(t_ad[i]));
+  }
+  auto tile_step = [&](int j, auto par) __attribute__((always_inline)) {
+    constexpr int stage = decltype(par)::value;
     const bool has_next = j + 1 < ntiles;
 
     const int key0 = j * kDqKV;
@@ -597,8 +605,8 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       auto load_kv = [&](int s, int buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-          kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kDqRowB + (k_rd ^ (s << 5)));
-          vf[buf][kb] = *reinterpret_cast<const bf16x8 *>(vt + kb * 32 * kDqRowB + (k_rd ^ (s << 5)));
+          kf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kb * 32 * kDqRowB));
+          vf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kDqTile + kb * 32 * kDqRowB));
         }
       };
 #pragma unroll
@@ -648,9 +656,9 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       constexpr int kPfT = 4;
       bf16x4 ktf[kPfT][2];
       auto load_t = [&](int u, int buf) {  // u = 4*t + db
-        const uint8_t *kp = kt + 16 * (u >> 2) * kDqRowB;
-        ktf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(kp + (t_rd ^ ((u & 3) << 5))));
-        ktf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(kp + 8 * kDqRowB + (t_rd ^ ((u & 3) << 5) ^ 16)));
+        const uint32_t ko = stage * kDqStage + 16 * (u >> 2) * kDqRowB;
+        ktf[buf][0] = lds_read_tr(lds_ptr(t_ad[u & 3] + ko));
+        ktf[buf][1] = lds_read_tr(lds_ptr(t_ad[4 + (u & 3)] + ko + 8 * kDqRowB));
       };
 #pragma unroll
       for (int u = 0; u < kPfT; ++u) load_t(u, u);
@@ -665,6 +673,10 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     }
     wait_vm0();
     __syncthreads();
+  };
+  for (int j = 0; j < ntiles; j += 2) {
+    tile_step(j, std::integral_constant<int, 0>{});
+    if (j + 1 < ntiles) tile_step(j + 1, std::integral_constant<int, 1>{});
   }
 
   // ---- epilogue: dQ rows (bf16)

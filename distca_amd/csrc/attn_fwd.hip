@@ -22,6 +22,7 @@
 // K/V tiles go from global memory straight into LDS (LDS-direct loads, four 256-byte rows per
 // instruction, rows unpadded with swizzled 16-byte chunks, see tile_swz), one period ahead of
 // their use.
+#include <type_traits>
 #include "api_util.h"
 #include "attn_cfg.h"
 #include "common.h"
@@ -160,11 +161,11 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
 #pragma unroll
     for (int i = 0; i < kLdW; ++i) lds_direct_load16(tb, voff[i], lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
   };
-  auto issue_k = [&](int j) {
+  auto issue_k = [&](int j) __attribute__((always_inline)) {
     if ((j + 1) * kFwdKV <= lk) issue_rows_fast(kbase, j, kKOff + (j & 1) * kKTile);
     else issue_rows(kbase, j, kKOff + (j & 1) * kKTile);
   };
-  auto issue_v = [&](int j) {
+  auto issue_v = [&](int j) __attribute__((always_inline)) {
     if ((j + 1) * kFwdKV <= lk) issue_rows_fast(vbase, j, kVOff + (j & 1) * kVTile);
     else issue_rows(vbase, j, kVOff + (j & 1) * kVTile);
   };
@@ -191,13 +192,22 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
   const int v_rd = (4 * g + i4) * kRowB + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*db ^ 16*hi
 
+  // Absolute LDS addresses of this lane's operand reads in stage 0, the eight swizzled variants of each,
+  // kept in registers: with the stage and the row block in the instruction's offset field, no address
+  // arithmetic is left between the MFMAs.
+  uint32_t k_ad[8], v_ad[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    k_ad[i] = lds0 + kKOff + (k_rd ^ (i << 5));
+    v_ad[i] = lds0 + kVOff + (v_rd ^ ((i & 3) << 5) ^ ((i >> 2) << 4));
+    asm volatile("" : "+v"(k_ad[i]), "+v"(v_ad[i]));
+  }
   f32x16 sacc[MSUB][2];
   bf16x8 pf[MSUB][4];
   auto tile_active = [&](int j) { return wave_live && j * kFwdKV <= lim_last; };
 
   // ---- S^T = K Q^T : [64 keys] x [32*MSUB rows]
-  auto phase_s = [&](int j) {
-    const uint8_t *kt = lds + kKOff + (j & 1) * kKTile;
+  auto phase_s = [&](int j, auto par) __attribute__((always_inline)) {  // par: parity of j, known at compile time
 #pragma unroll
     for (int m = 0; m < MSUB; ++m)
 #pragma unroll
@@ -208,7 +218,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     bf16x8 kf[kPf][2];
     auto load_k = [&](int s, int buf) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *reinterpret_cast<const bf16x8 *>(kt + kb * 32 * kRowB + (k_rd ^ (s << 5)));
+      for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + decltype(par)::value * kKTile + kb * 32 * kRowB));
     };
 #pragma unroll
     for (int s = 0; s < kPf; ++s) load_k(s, s);
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     }
   };
   // ---- mask, online softmax (log2 domain, one query row per lane pair), P as bf16 B operand
-  auto phase_x = [&](int j) {
+  auto phase_x = [&](int j) __attribute__((always_inline)) {
     const int key0 = j * kFwdKV;
     if (key0 + kFwdKV - 1 > lim_first) {  // the tile straddles the diagonal or the end of the prefix
 #pragma unroll
@@ -290,14 +300,13 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     }
   };
   // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
-  auto phase_pv = [&](int j) {
-    const uint8_t *vt = lds + kVOff + (j & 1) * kVTile;
+  auto phase_pv = [&](int j, auto par) __attribute__((always_inline)) {
     constexpr int kPfV = 4;  // V^T fragments are requested four MFMAs ahead
     bf16x4 vf[kPfV][2];
     auto load_v = [&](int u, int buf) {  // u = 4*t + db
-      const uint8_t *vp = vt + 16 * (u >> 2) * kRowB;
-      vf[buf][0] = lds_read_tr((const DISTCA_LDS void *)(vp + (v_rd ^ ((u & 3) << 5))));
-      vf[buf][1] = lds_read_tr((const DISTCA_LDS void *)(vp + 8 * kRowB + (v_rd ^ ((u & 3) << 5) ^ 16)));
+      const uint32_t vo = decltype(par)::value * kVTile + 16 * (u >> 2) * kRowB;
+      vf[buf][0] = lds_read_tr(lds_ptr(v_ad[u & 3] + vo));
+      vf[buf][1] = lds_read_tr(lds_ptr(v_ad[4 + (u & 3)] + vo + 8 * kRowB));
     };
 #pragma unroll
     for (int u = 0; u < kPfV; ++u) load_v(u, u);
@@ -326,29 +335,45 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   if (ntiles > 0) issue_k(0);
   wait_vm0();
   __syncthreads();  // b0
+  // The period loop is unrolled by two so that the LDS stage of every operand read is a constant folded into
+  // the instruction's offset field instead of an addition per read between the MFMAs.
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  auto period0 = [&](int p, auto par) __attribute__((always_inline)) {   // par = parity of p
+    using Same = std::integral_constant<int, decltype(par)::value>;
+    using Other = std::integral_constant<int, 1 - decltype(par)::value>;
+    if (p > 0 && tile_active(p - 1)) phase_pv(p - 1, Other{});
+    const bool act = p < ntiles && tile_active(p);
+    if (act) phase_s(p, Same{});
+    __syncthreads();
+    if (p + 1 < ntiles) issue_k(p + 1);
+    if (p < ntiles) issue_v(p);
+    if (act) phase_x(p);
+    wait_vm0();
+    __syncthreads();
+  };
+  auto period1 = [&](int p, auto par) __attribute__((always_inline)) {
+    using Same = std::integral_constant<int, decltype(par)::value>;
+    using Other = std::integral_constant<int, 1 - decltype(par)::value>;
+    if (p + 1 < ntiles) issue_k(p + 1);
+    if (p < ntiles) issue_v(p);
+    const bool act_prev = p > 0 && tile_active(p - 1);
+    if (act_prev) phase_x(p - 1);
+    __syncthreads();
+    if (act_prev) phase_pv(p - 1, Other{});
+    if (p < ntiles && tile_active(p)) phase_s(p, Same{});
+    wait_vm0();
+    __syncthreads();
+  };
   if (grp == 0) {
-    for (int p = 0; p <= ntiles; ++p) {
-      if (p > 0 && tile_active(p - 1)) phase_pv(p - 1);
-      const bool act = p < ntiles && tile_active(p);
-      if (act) phase_s(p);
-      __syncthreads();
-      if (p + 1 < ntiles) issue_k(p + 1);
-      if (p < ntiles) issue_v(p);
-      if (act) phase_x(p);
-      wait_vm0();
-      __syncthreads();
+    for (int p = 0; p <= ntiles; p += 2) {
+      period0(p, P0{});
+      if (p + 1 <= ntiles) period0(p + 1, P1{});
     }
   } else {
-    for (int p = 0; p <= ntiles; ++p) {
-      if (p + 1 < ntiles) issue_k(p + 1);
-      if (p < ntiles) issue_v(p);
-      const bool act_prev = p > 0 && tile_active(p - 1);
-      if (act_prev) phase_x(p - 1);
-      __syncthreads();
-      if (act_prev) phase_pv(p - 1);
-      if (p < ntiles && tile_active(p)) phase_s(p);
-      wait_vm0();
-      __syncthreads();
+    for (int p = 0; p <= ntiles; p += 2) {
+      period1(p, P0{});
+      if (p + 1 <= ntiles) period1(p + 1, P1{});
     }
   }
 

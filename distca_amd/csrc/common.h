@@ -35,6 +35,8 @@ __device__ __forceinline__ constexpr int acc_row(int r, int g) { return 8 * (r >
 // chunks supplied by lanes 4e + L/4, e = 0..3.  With lane j pointing at
 // (row r0 + j/4, col c0 + 4*(j%4)) of a row-major tile, lane L ends up with
 // column c0 + L of rows r0 .. r0+3.
+// An LDS pointer from a 32-bit LDS address.
+__device__ __forceinline__ const DISTCA_LDS void *lds_ptr(uint32_t addr) { return reinterpret_cast<const DISTCA_LDS void *>(static_cast<uintptr_t>(addr)); }
 __device__ __forceinline__ bf16x4 lds_read_tr(const DISTCA_LDS void *p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DISTCA_LDS s16x4 *)p);
   return __builtin_bit_cast(bf16x4, v);
