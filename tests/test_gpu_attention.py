@@ -9,7 +9,7 @@ from oracle.attention import ca_reference_bwd, ca_reference_fwd
 pytestmark = pytest.mark.gpu
 
 
-def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128):
+def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128, kv_grad_tol=None):
     from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
     cu_q, cu_k = cu(q_lens), cu(k_lens)
     tq = int(cu_q[-1])
@@ -37,8 +37,9 @@ def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, tota
                                False, dkv)
     torch.cuda.synchronize()
     assert_close_bf16(dq, ref_dq, "dq")
-    assert_close_bf16(dk, ref_dk, "dk")
-    assert_close_bf16(dv, ref_dv, "dv")
+    tol = dict(max_abs=kv_grad_tol[0], mean_rel=kv_grad_tol[1]) if kv_grad_tol else {}
+    assert_close_bf16(dk, ref_dk, "dk", **tol)
+    assert_close_bf16(dv, ref_dv, "dv", **tol)
 
 
 def test_config1_tiny_forward(cuda):
@@ -55,10 +56,13 @@ def test_whole_docs_fwd_bwd_medium(cuda):
     _run([512, 1024, 700], [512, 1024, 700], 32, 8, 2, cuda)
 
 
-@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 1), (6, 2), (16, 2)])
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 1), (6, 2), (16, 2), (64, 1), (24, 8), (32, 1)])
 def test_head_groupings(cuda, hq, hkv):
-    """MHA, MQA, a non-power-of-two group and the Llama-3-70B group of 8."""
-    _run([300, 45], [300, 45], hq, hkv, 3, cuda)
+    """MHA, MQA, a non-power-of-two group, the Llama-3-70B group of 8; groups of 64 (more heads per token than a
+    backward row block holds), of 3 (a row block does not start at a token boundary) and of 32 (exactly one)."""
+    # dK and dV of a kv head sum the bf16-rounded P and dS of all its query heads: with 32 or 64 of them the
+    # rounding noise of the sum (growing as the square root of the count) is allowed twice the bar
+    _run([300, 45], [300, 45], hq, hkv, 3, cuda, kv_grad_tol=(4e-2, 2e-3) if hq // hkv >= 32 else None)
 
 
 def test_prefix_tasks_lk_gt_lq(cuda):
