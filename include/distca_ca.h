@@ -120,6 +120,12 @@ typedef struct distca_ca_params {
   int32_t reserved;
 } distca_ca_params;
 
+/* Size of the workspace an attention call needs (no reference counterpart: flash-attn
+ * allocates its own).  The workspace holds the work list the call builds on the device
+ * and the counters its workgroups draw their work from (and, in the backward, the row
+ * statistics and the fp32 accumulators of aliased K/V rows); its contents are rewritten
+ * by every call, so calls that may run at the same time on different streams each need
+ * a workspace of their own, while calls ordered on one stream can share one.           */
 int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p);
 int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p);
 
