@@ -205,3 +205,20 @@ def test_token_layout_entry_points_check_their_layouts():
     p = idle
     assert fwd(q=None, q_off=None, k=None, v=None, out=None, out_off=None, cu_q=None, cu_k=None, ws=None, ws_bytes=0) == 0
     p = p_save
+
+
+def test_torch_ops_are_registered_for_device_tensors_only():
+    """`torch.ops.distca_amd.*` carry the reference's op names and schemas
+    (csrc/bindings/all_to_all.cpp:102-113,182-254) and have no host implementation."""
+    import torch
+    from distca_amd import torch_ops
+    for name, schema in torch_ops.SCHEMAS.items():
+        op = getattr(torch.ops.distca_amd, name)
+        got = str(op.default._schema)
+        assert got == f"distca_amd::{name}{schema}", got
+    t = torch.zeros((4, 8), dtype=torch.bfloat16)
+    i64 = torch.zeros(1, dtype=torch.int64)
+    with pytest.raises(NotImplementedError):
+        torch.ops.distca_amd.fast_a2a_memcpy_non_cp_debug(t, i64, i64, None, True, torch.zeros(64, dtype=torch.uint8))
+    with pytest.raises(NotImplementedError):
+        torch.ops.distca_amd.fast_a2a_grad_acc(t, torch.zeros(1, dtype=torch.int32), torch.zeros((1, 1), dtype=torch.int64), i64)

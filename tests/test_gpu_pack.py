@@ -123,3 +123,56 @@ def test_grad_sum(cuda, dtype, hidden):
     pre_a2a_grad_acc(d, torch.from_numpy(nc_arr).to(cuda), torch.from_numpy(cs).to(cuda), torch.tensor(lens, dtype=torch.int64, device=cuda))
     torch.cuda.synchronize()
     assert torch.equal(d.cpu().view(torch.uint8), exp.view(torch.uint8))
+
+
+def test_through_torch_ops(cuda):
+    """The same kernels called as `torch.ops.distca_amd.*` with the reference's op names and argument
+    order (csrc/bindings/all_to_all.cpp:102-113,182-254): pack, replicating pack and duplicate sum."""
+    from distca_amd import torch_ops  # noqa: F401  (registers the ops)
+    rng = np.random.default_rng(5)
+    nshard, hidden = 6, 256
+    lens = rng.integers(1, 30, size=nshard).astype(np.int64)
+    T, tb = int(lens.sum()), hidden * 2
+    off, nbuf = _layout(rng, lens, tb)
+    src = torch.from_numpy(rng.integers(0, 256, size=(T, tb), dtype=np.uint8))
+    mask = np.array([1, 0, 1, 1, 0, 1], dtype=np.int8)
+    exp = np.full(nbuf, 0x33, dtype=np.uint8)
+    fa2a.copy_non_cp(src.numpy(), exp, off, lens, mask, True)
+    dbuf = torch.full((nbuf,), 0x33, dtype=torch.uint8, device=cuda)
+    d_off, d_len = torch.from_numpy(off).to(cuda), torch.from_numpy(lens).to(cuda)
+    print("torch.ops non_cp", flush=True)
+    torch.ops.distca_amd.fast_a2a_memcpy_non_cp_debug(src.view(torch.bfloat16).to(cuda), d_off, d_len, torch.from_numpy(mask).to(cuda), True, dbuf)
+    torch.cuda.synchronize()
+    assert np.array_equal(dbuf.cpu().numpy(), exp)
+
+    max_cp = 2
+    do_shard = np.ones((nshard, max_cp), dtype=np.int8)
+    do_shard[2, 1] = 0
+    off2 = np.zeros((max_cp, nshard), dtype=np.int64)
+    cur = 0
+    for c in range(max_cp):
+        for s in rng.permutation(nshard):
+            off2[c, s] = cur
+            cur += int(lens[s]) * tb
+    exp2 = np.zeros(cur, dtype=np.uint8)
+    fa2a.copy_cp(src.numpy(), exp2, do_shard, off2, lens, True)
+    dbuf2 = torch.zeros(cur, dtype=torch.uint8, device=cuda)
+    print("torch.ops cp", flush=True)
+    torch.ops.distca_amd.fast_a2a_memcpy_cp_debug(src.view(torch.bfloat16).to(cuda), torch.from_numpy(do_shard).to(cuda),
+                                                  torch.from_numpy(off2).to(cuda), d_len, True, dbuf2)
+    torch.cuda.synchronize()
+    assert np.array_equal(dbuf2.cpu().numpy(), exp2)
+
+    # rows 0..9 are a main shard with one copy in rows 10..19
+    g = torch.Generator().manual_seed(9)
+    data = torch.randn((20, hidden), generator=g).to(torch.bfloat16)
+    nc = np.array([1, 0], dtype=np.int32)
+    cs = np.array([[10], [0]], dtype=np.int64)
+    ln = [10, 10]
+    expd = data.clone()
+    fa2a.grad_sum(expd, nc, cs, ln)
+    d = data.to(cuda)
+    print("torch.ops grad_acc", flush=True)
+    torch.ops.distca_amd.fast_a2a_grad_acc(d, torch.from_numpy(nc).to(cuda), torch.from_numpy(cs).to(cuda), torch.tensor(ln, dtype=torch.int64, device=cuda))
+    torch.cuda.synchronize()
+    assert torch.equal(d.cpu().view(torch.uint8), expd.view(torch.uint8))
