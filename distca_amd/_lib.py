@@ -13,7 +13,7 @@ from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int6
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdistca_ca.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class CaParams(Structure):

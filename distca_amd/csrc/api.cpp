@@ -88,4 +88,4 @@ extern "C" int distca_timing_read(int which, double *total_ms, int64_t *launches
 }
 
 extern "C" const char *distca_last_error(void) { return distca::error_buffer(); }
-extern "C" int distca_abi_version(void) { return 2; }
+extern "C" int distca_abi_version(void) { return 3; }

@@ -122,7 +122,18 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     if (t_first < 0) t_first = 0;
     mb0 = (int)(((int64_t)t_first * G) / kBM);
   }
-  const int niter = nmb > mb0 ? nmb - mb0 : 0;
+  // the query blocks of this item, visited from block top - 1 down to block bot: all that see the key block,
+  // or one piece of them (sched.h)
+  int top = nmb, bot = mb0;
+  {
+    const int piece = it4.w & 0xffff, pieces = it4.w >> 16;
+    if (pieces > 1) {
+      const int n = nmb > mb0 ? nmb - mb0 : 0;
+      top = nmb - piece_begin(n, piece, pieces);
+      bot = nmb - piece_begin(n, piece + 1, pieces);
+    }
+  }
+  const int niter = top > bot ? top - bot : 0;
 
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
@@ -184,7 +195,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   auto issue_tile = [&](int stage, int mbx) {
     const int tile = kTileOff + stage * kTileBytes;
     const int stat = kStatOff + stage * kStatBytes;
-    const bool blk_ok = mbx >= mb0;
+    const bool blk_ok = mbx >= bot;
     if (fast_ok && blk_ok && (mbx + 1) * kBM <= nrows) {
       const int tok0 = mbx * tok_per_blk;
       if (lane < 4) {
@@ -364,15 +375,15 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
   __syncthreads();  // K has left LDS: its region now holds the tile ring
   if (niter > 0) {
-    issue_tile(0, nmb - 1);
-    issue_tile(1, nmb - 2);
+    issue_tile(0, top - 1);
+    issue_tile(1, top - 2);
   }
   wait_vm0();
   if (grp == 0) {
     for (int p = 0; p < niter; ++p) {
       wait_older();
       __syncthreads();  // b1(p): tile p is complete
-      issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      issue_tile((p + 2) % kStages, top - 1 - (p + 2));
       __builtin_amdgcn_s_setprio(3);
       phase_a(p % kStages);
       __builtin_amdgcn_s_setprio(0);
@@ -387,7 +398,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     __syncthreads();    // b1(0)
     for (int p = 0; p < niter; ++p) {
       __syncthreads();  // b2(p)
-      issue_tile((p + 2) % kStages, nmb - 1 - (p + 2));
+      issue_tile((p + 2) % kStages, top - 1 - (p + 2));
       __builtin_amdgcn_s_setprio(3);
       phase_a(p % kStages);
       __builtin_amdgcn_s_setprio(0);
@@ -402,27 +413,48 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   wait_vm0();  // nothing may still be on its way into LDS when the workgroup ends
 
   // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
-  const int key = kw0 + l32;
-  if (key < lk) {
-    const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
+  if (ALIAS) {
+    // Work items that share K/V rows (tasks over one stored prefix, pieces of one key block) add up in
+    // fp32; the order of these additions is the one source of run-to-run variation.  A lane holds one key's
+    // values, 2 KB apart from its neighbour's in memory: the sums pass through LDS so that one atomic
+    // instruction covers 64 consecutive floats of a row instead of 64 rows.
+    constexpr int kEpiPitch = (kHeadDim + 4) * 4;  // bytes per key row in LDS; the 16 spare bytes spread the banks
+    static_assert(kBN * kEpiPitch <= kBwdLds, "the epilogue stages one 256 x 128 fp32 matrix in LDS");
+    const int wkey0 = (grp * 4 + kbw) * 32;        // this wave's rows of the staging matrix: written and read by it alone
+    const int nkeys = lk - kw0 < 32 ? lk - kw0 : 32;
+    __syncthreads();                               // every wave has finished with the V tile and the tile ring
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int which = 0; which < 2; ++which) {
+      float *dst = which == 0 ? a.dk_acc : a.dv_acc;
 #pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-        if (ALIAS) {
-          // tasks that share KV rows add up here; the order of these additions is the one
-          // source of run-to-run variation, and only in the aliased-prefix form
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            unsafeAtomicAdd(a.dk_acc + off + d0 + rr, dkacc[db][4 * cq + rr]);
-            unsafeAtomicAdd(a.dv_acc + off + d0 + rr, dvacc[db][4 * cq + rr]);
-          }
-        } else {
+        for (int cq = 0; cq < 4; ++cq) {
+          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
+          const f32x16 &acc = which == 0 ? dkacc[db] : dvacc[db];
+          *reinterpret_cast<f32x4 *>(lds + (wkey0 + l32) * kEpiPitch + d0 * 4) = f32x4{acc[4 * cq], acc[4 * cq + 1], acc[4 * cq + 2], acc[4 * cq + 3]};
+        }
+      // LDS operations of one wave complete in order: the reads below see the writes above
+      for (int kk = 0; kk < nkeys; ++kk) {
+        const float *row = reinterpret_cast<const float *>(lds + (wkey0 + kk) * kEpiPitch);
+        float *out = dst + (int64_t)(ks + kw0 + kk) * kv_stride + kvh * kHeadDim;
+        unsafeAtomicAdd(out + lane, row[lane]);
+        unsafeAtomicAdd(out + 64 + lane, row[64 + lane]);
+      }
+    }
+  } else {
+    const int key = kw0 + l32;
+    if (key < lk) {
+      const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int cq = 0; cq < 4; ++cq) {
+          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
           *reinterpret_cast<bf16x4 *>(a.dk + off + d0) = cvt4(dkacc[db][4 * cq], dkacc[db][4 * cq + 1], dkacc[db][4 * cq + 2], dkacc[db][4 * cq + 3]);
           *reinterpret_cast<bf16x4 *>(a.dv + off + d0) = cvt4(dvacc[db][4 * cq], dvacc[db][4 * cq + 1], dvacc[db][4 * cq + 2], dvacc[db][4 * cq + 3]);
         }
-      }
+    }
   }
 }
 
@@ -860,7 +892,9 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
   }
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
     return fail(DISTCA_E_INVALID, "ca_bwd: tensors must be 16-byte aligned");
-  const BwdWorkspace w = bwd_layout(p, alias);
+  // dK/dV go through fp32 accumulators when tasks alias K/V rows or when key blocks are cut into pieces
+  const bool use_acc = alias || bwd_split_target(p) > 0;
+  const BwdWorkspace w = bwd_layout(p, use_acc);
   if (!workspace || workspace_bytes < w.total)
     return fail(DISTCA_E_WORKSPACE, "ca_bwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)w.total);
   if (!aligned16(workspace)) return fail(DISTCA_E_INVALID, "ca_bwd: workspace must be 16-byte aligned");
@@ -871,7 +905,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
 
   // rows no task touches must come back as zero
   if (kv_elems > 0) {
-    if (alias) {
+    if (use_acc) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 2)), dim3(256), 0, s, (u32x4 *)(ws + w.dk_acc),
                          (w.total - w.dk_acc) / 16);
     } else {
@@ -891,8 +925,8 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
   a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta);
   a.dq = (__bf16 *)dq; a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
   a.qs_task_off = qs.task_off; a.qs_tok_bytes = qs.tok_bytes; a.dq_task_off = qs.dq_task_off; a.dq_tok_bytes = qs.dq_tok_bytes;
-  a.dk_acc = alias ? (float *)(ws + w.dk_acc) : nullptr;
-  a.dv_acc = alias ? (float *)(ws + w.dv_acc) : nullptr;
+  a.dk_acc = use_acc ? (float *)(ws + w.dk_acc) : nullptr;
+  a.dv_acc = use_acc ? (float *)(ws + w.dv_acc) : nullptr;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
@@ -920,7 +954,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
-    if (alias)
+    if (use_acc)
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
     else
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
@@ -939,7 +973,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
     hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
   }
-  if (alias) {
+  if (use_acc) {
     hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (__bf16 *)dk, kv_elems / 8);
     hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dv_acc), (__bf16 *)dv, kv_elems / 8);
   }

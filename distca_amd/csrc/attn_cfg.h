@@ -49,12 +49,32 @@ inline int validate_params(const distca_ca_params *p) {
 
 inline SchedGeom fwd_geom(const distca_ca_params *p) {
   SchedGeom g;
+  g.split_target = 0;
   g.rows_per_block = kFwdRows;
   g.kv_per_block = kFwdKV;
   g.group = p->num_heads_q / p->num_heads_kv;
   g.causal = p->causal != 0;
   g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_k / kFwdKV + 1);
   return g;
+}
+// Compute units of the device this library is built for (MI355X).
+constexpr int kNumCUs = 256;
+// Key blocks are cut into pieces (sched.h) when the batch has so few of them that they could not occupy the
+// device twice over, unless the caller asked for a deterministic backward (the pieces' dK/dV are added up with
+// float atomics).  Returns the number of pieces to aim for per kv head, 0 = no cutting.
+constexpr int kSplitPiecesPerCU = 2;
+inline int64_t bwd_key_blocks_bound(const distca_ca_params *p) {
+  // sum over tasks of ceil(Lk / kBwdKV); sum of Lk may exceed total_k when prefixes alias,
+  // but each Lk <= max_seqlen_k.
+  const int64_t by_total = (int64_t)p->total_k / kBwdKV + p->num_tasks + 1;
+  const int64_t by_max = ((int64_t)p->max_seqlen_k / kBwdKV + 1) * p->num_tasks + 1;
+  return by_total > by_max ? by_total : by_max;
+}
+inline int32_t bwd_split_target(const distca_ca_params *p) {
+  if (p->deterministic) return 0;
+  if (bwd_key_blocks_bound(p) * p->num_heads_kv >= 2 * kNumCUs) return 0;
+  const int32_t t = kSplitPiecesPerCU * kNumCUs / p->num_heads_kv;
+  return t > 0 ? t : 1;
 }
 inline SchedGeom dq_geom(const distca_ca_params *p) {
   SchedGeom g = fwd_geom(p);
@@ -68,6 +88,7 @@ inline SchedGeom bwd_geom(const distca_ca_params *p) {
   g.group = p->num_heads_q / p->num_heads_kv;
   g.causal = p->causal != 0;
   g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_q * g.group / kBwdRows + 1);
+  g.split_target = bwd_split_target(p);
   return g;
 }
 // Upper bound of the item count that needs only host-known sizes.
@@ -80,11 +101,8 @@ inline int64_t dq_max_items(const distca_ca_params *p) {
   return (int64_t)p->total_q * group / kDqRows + p->num_tasks + 1;
 }
 inline int64_t bwd_max_items(const distca_ca_params *p) {
-  // sum over tasks of ceil(Lk / kBwdKV); sum of Lk may exceed total_k when prefixes alias,
-  // but each Lk <= max_seqlen_k.
-  const int64_t by_total = (int64_t)p->total_k / kBwdKV + p->num_tasks + 1;
-  const int64_t by_max = ((int64_t)p->max_seqlen_k / kBwdKV + 1) * p->num_tasks + 1;
-  return by_total > by_max ? by_total : by_max;
+  // cutting adds at most total cost / piece <= split_target pieces to the key blocks
+  return bwd_key_blocks_bound(p) + bwd_split_target(p);
 }
 
 int launch_build_schedule(int kind, const int32_t *cu_q, const int32_t *cu_k, int32_t num_tasks, const SchedGeom &g,

@@ -27,7 +27,24 @@ struct SchedGeom {
   int32_t group;           // Hq / Hkv
   int32_t causal;
   int32_t cost_shift;      // bin = min(kSchedBins-1, cost >> cost_shift)
+  int32_t split_target;    // backward only, 0 = off: cut expensive key blocks into pieces so that about this
+                           // many pieces exist per kv head (see piece_count)
 };
+
+// Cutting key blocks: a batch of few tokens has fewer key blocks than the device has compute units, and
+// the block at the start of a long document streams every query row below it, so without cuts the launch
+// lasts as long as that one workgroup.  A block of cost c (query blocks to stream) is cut into
+// ceil(c / piece) pieces of consecutive query blocks, piece = max(kMinPiece, total cost / split_target);
+// the pieces are independent work items whose dK/dV are added up in fp32.
+constexpr int32_t kMinPiece = 16;
+constexpr int32_t kMaxPieces = 64;
+DISTCA_HD int32_t piece_count(int32_t cost, int32_t piece) {
+  if (piece <= 0) return 1;
+  int32_t k = (cost + piece - 1) / piece;
+  return k < 1 ? 1 : (k > kMaxPieces ? kMaxPieces : k);
+}
+// query blocks [lo, hi) of piece j of k over n blocks, counted from the last block downwards
+DISTCA_HD int32_t piece_begin(int32_t n, int32_t j, int32_t k) { return (int32_t)(((int64_t)n * j) / k); }
 
 constexpr int kSchedBins = 4096;
 
@@ -77,7 +94,7 @@ inline int32_t pick_cost_shift(int64_t max_cost) {
 
 // Workspace layout of a schedule (all int32):
 //   [0] item count   [1..3] reserved   [4 .. 4+B] exclusive block prefix per task
-//   then items as (task, block, cost, 0) quadruples, 16-byte aligned.
+//   then items as (task, block, cost, piece | pieces << 16) quadruples, 16-byte aligned.
 DISTCA_HD int64_t sched_header_ints(int32_t num_tasks) { return ((int64_t)4 + num_tasks + 1 + 3) / 4 * 4; }
 DISTCA_HD int64_t sched_bytes(int32_t num_tasks, int64_t max_items) {
   return (sched_header_ints(num_tasks) + 4 * max_items) * (int64_t)sizeof(int32_t);

@@ -75,11 +75,29 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
   for (int i = tid; i < kSchedBins; i += kSchedThreads) bins[i] = 0;
   __syncthreads();
 
+  // 1b. (backward, when asked for) the piece size that cuts expensive key blocks
+  __shared__ unsigned long long total_cost;
+  int32_t piece = 0;
+  if (BWD && g.split_target > 0) {
+    if (tid == 0) total_cost = 0;
+    __syncthreads();
+    unsigned long long local = 0;
+    for (int32_t e = tid; e < nitems; e += kSchedThreads) {
+      const int32_t b = find_task(base, num_tasks, e);
+      local += (unsigned long long)item_cost<BWD>(g, cu_q, cu_k, b, e - base[b]);
+    }
+    atomicAdd(&total_cost, local);
+    __syncthreads();
+    const unsigned long long per = total_cost / (unsigned long long)g.split_target;
+    piece = per > (unsigned long long)kMinPiece ? (int32_t)(per < 0x7fffffffull ? per : 0x7fffffffull) : kMinPiece;
+  }
+
   // 2. histogram of cost bins
   for (int32_t e = tid; e < nitems; e += kSchedThreads) {
     const int32_t b = find_task(base, num_tasks, e);
     const int32_t cost = item_cost<BWD>(g, cu_q, cu_k, b, e - base[b]);
-    atomicAdd(&bins[cost_bin(g, cost)], 1);
+    const int32_t k = piece_count(cost, piece);
+    for (int32_t j = 0; j < k; ++j) atomicAdd(&bins[cost_bin(g, piece_begin(cost, j + 1, k) - piece_begin(cost, j, k))], 1);
   }
   __syncthreads();
 
@@ -108,14 +126,21 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
     const int32_t b = find_task(base, num_tasks, e);
     const int32_t i = e - base[b];
     const int32_t cost = item_cost<BWD>(g, cu_q, cu_k, b, i);
-    const int32_t pos = atomicAdd(&bins[cost_bin(g, cost)], 1);
-    if (pos < max_items) {
-      int4 it = make_int4(b, i, cost, 0);
-      reinterpret_cast<int4 *>(items)[pos] = it;
+    const int32_t k = piece_count(cost, piece);
+    for (int32_t j = 0; j < k; ++j) {
+      const int32_t cj = piece_begin(cost, j + 1, k) - piece_begin(cost, j, k);
+      const int32_t pos = atomicAdd(&bins[cost_bin(g, cj)], 1);
+      if (pos < max_items) {
+        int4 it = make_int4(b, i, cj, j | (k << 16));
+        reinterpret_cast<int4 *>(items)[pos] = it;
+      }
     }
   }
+  __syncthreads();
   if (tid == 0) {
-    ws[0] = nitems;
+    // after the scatter the counter of the cheapest bin holds the number of entries
+    const int32_t total = bins[0];
+    ws[0] = total < max_items ? total : max_items;
     ws[1] = running;
   }
   if (tid < kZeroRowBytes / 4) ws[sched_zero_row_off(num_tasks, max_items) / 4 + tid] = 0;
@@ -157,22 +182,37 @@ extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const 
   if (rc) return rc;
   if (kind != 0 && kind != 1) return fail(DISTCA_E_INVALID, "schedule_host: kind must be 0 (fwd) or 1 (bwd)");
   const SchedGeom g = kind == 0 ? fwd_geom(p) : bwd_geom(p);
-  struct It { int32_t task, block, cost, bin; };
-  std::vector<It> v;
+  struct It { int32_t task, block, cost, bin, piece; };
+  std::vector<It> whole, v;
+  unsigned long long total_cost = 0;
   for (int32_t b = 0; b < p->num_tasks; ++b) {
     const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
     const int32_t n = kind == 0 ? fwd_num_blocks(g, lq) : bwd_num_blocks(g, lq, lk);
     for (int32_t i = 0; i < n; ++i) {
       const int32_t c = kind == 0 ? fwd_cost(g, lq, lk, i) : bwd_cost(g, lq, lk, i);
-      v.push_back({b, i, c, cost_bin(g, c)});
+      whole.push_back({b, i, c, 0, 0});
+      total_cost += (unsigned long long)c;
+    }
+  }
+  int32_t piece = 0;
+  if (kind == 1 && g.split_target > 0) {
+    const unsigned long long per = total_cost / (unsigned long long)g.split_target;
+    piece = per > (unsigned long long)kMinPiece ? (int32_t)(per < 0x7fffffffull ? per : 0x7fffffffull) : kMinPiece;
+  }
+  for (const It &w : whole) {
+    const int32_t k = piece_count(w.cost, piece);
+    for (int32_t j = 0; j < k; ++j) {
+      const int32_t cj = piece_begin(w.cost, j + 1, k) - piece_begin(w.cost, j, k);
+      v.push_back({w.task, w.block, cj, cost_bin(g, cj), j | (k << 16)});
     }
   }
   std::stable_sort(v.begin(), v.end(), [](const It &a, const It &b) { return a.bin > b.bin; });
   const int64_t n = (int64_t)v.size();
   for (int64_t e = 0; e < n && e < max_items; ++e) {
-    items[3 * e + 0] = v[e].task;
-    items[3 * e + 1] = v[e].block;
-    items[3 * e + 2] = v[e].cost;
+    items[4 * e + 0] = v[e].task;
+    items[4 * e + 1] = v[e].block;
+    items[4 * e + 2] = v[e].cost;
+    items[4 * e + 3] = v[e].piece;
   }
   return n;
 }

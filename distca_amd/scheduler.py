@@ -17,13 +17,13 @@ from . import _lib
 FWD, BWD = 0, 1
 
 
-def _params(cu_q, cu_k, hq, hkv, d, causal) -> _lib.CaParams:
+def _params(cu_q, cu_k, hq, hkv, d, causal, deterministic=False) -> _lib.CaParams:
     cu_q = np.asarray(cu_q, dtype=np.int64)
     cu_k = np.asarray(cu_k, dtype=np.int64)
     lq, lk = np.diff(cu_q), np.diff(cu_k)
     return _lib.CaParams(len(lq), int(cu_q[-1]), int(cu_k[-1]), hq, hkv, d,
                          int(lq.max()) if len(lq) else 0, int(lk.max()) if len(lk) else 0,
-                         float(d) ** -0.5, 1 if causal else 0, 0, 0)
+                         float(d) ** -0.5, 1 if causal else 0, 1 if deterministic else 0, 0)
 
 
 def tile_shape(kind: int, hq: int, hkv: int, d: int = 128) -> Tuple[int, int]:
@@ -35,17 +35,28 @@ def tile_shape(kind: int, hq: int, hkv: int, d: int = 128) -> Tuple[int, int]:
 
 
 def build_schedule(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequence[int], num_heads_q: int,
-                   num_heads_kv: int, head_dim: int = 128, causal: bool = True) -> np.ndarray:
-    """Work items as an int32 array [n, 3] of (task, block, cost), most expensive first."""
+                   num_heads_kv: int, head_dim: int = 128, causal: bool = True, deterministic: bool = False) -> np.ndarray:
+    """Work items as an int32 array [n, 4] of (task, block, cost, piece | pieces << 16), most expensive
+    first.  Backward items of a batch too small to occupy the device are cut into pieces of
+    consecutive query blocks unless `deterministic`; everything else has pieces = 1, piece = 0."""
     cu_q = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
     cu_k = np.ascontiguousarray(cu_seqlens_k, dtype=np.int32)
-    p = _params(cu_q, cu_k, num_heads_q, num_heads_kv, head_dim, causal)
+    p = _params(cu_q, cu_k, num_heads_q, num_heads_kv, head_dim, causal, deterministic)
     lib = _lib.load()
     n = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), None, 0)
     if n < 0:
         _lib.check(int(n), "build_schedule")
-    items = np.zeros((int(n), 3), dtype=np.int32)
+    items = np.zeros((int(n), 4), dtype=np.int32)
     if n:
         m = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), items.ctypes.data, int(n))
         assert m == n
     return items
+
+
+def whole_items(items: np.ndarray) -> np.ndarray:
+    """[m, 3] (task, block, cost) with the pieces of every block put together again, most expensive first."""
+    total = {}
+    for t, b, c, _ in items.tolist():
+        total[(t, b)] = total.get((t, b), 0) + c
+    out = np.array([(t, b, c) for (t, b), c in total.items()], dtype=np.int32).reshape(-1, 3)
+    return out[np.argsort(-out[:, 2], kind="stable")] if len(out) else out

@@ -194,9 +194,11 @@ int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off,
  * host arrays so the balance invariants can be tested without a GPU.
  * kind 0 = forward (one item per (task, block of query rows), cost = KV tiles
  * visible to the block), 1 = backward (one item per (task, KV block), cost =
- * query blocks that see it).  Writes up to max_items (task, block, cost)
- * triples sorted by descending cost and returns the item count, or a negative
- * error.  The reference has no counterpart: flash-attn launches a static
+ * query blocks that see it; when the batch has too few key blocks to occupy
+ * the device and p->deterministic is 0, a key block is cut into pieces of
+ * consecutive query blocks, whose dK/dV the kernel adds up in fp32).  Writes
+ * up to max_items (task, block, cost, piece | pieces << 16) quadruples sorted
+ * by descending cost and returns the item count, or a negative error.  The reference has no counterpart: flash-attn launches a static
  * (m-block, batch, head) grid sized by max_seqlen_q.
  * ------------------------------------------------------------------------- */
 int64_t distca_ca_schedule_host(int kind, const int32_t *cu_seqlens_q,

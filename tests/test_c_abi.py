@@ -111,7 +111,7 @@ def test_schedule_host_reports_needed_capacity():
     p = _p(total_q=1000, total_k=1000, max_seqlen_q=1000, max_seqlen_k=1000)
     n = lib.distca_ca_schedule_host(0, cu.ctypes.data, cu.ctypes.data, ctypes.byref(p), None, 0)
     assert n > 0
-    small = np.full((2, 3), -7, dtype=np.int32)
+    small = np.full((2, 4), -7, dtype=np.int32)
     # a short array receives the first max_items items; the full count is still returned
     assert lib.distca_ca_schedule_host(0, cu.ctypes.data, cu.ctypes.data, ctypes.byref(p), small.ctypes.data, 1) == n
     assert small[0, 0] == 0 and (small[1] == -7).all()

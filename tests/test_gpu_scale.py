@@ -143,7 +143,7 @@ def test_prefix_tasks_equal_whole_document(cuda):
 @pytest.mark.parametrize("kind", ["fwd", "bwd"])
 def test_device_schedule_equals_host_mirror(cuda, kind):
     """The workspace begins with the schedule the device built ([0] = item count, then the
-    per-task block prefix, then (task, block, cost, 0) items): same items, same order of cost
+    per-task block prefix, then (task, block, cost, piece | pieces << 16) items): same items, same order of cost
     bins as distca_ca_schedule_host."""
     from distca_amd import scheduler, workloads
     from distca_amd._lib import CaParams, load
@@ -168,9 +168,7 @@ def test_device_schedule_equals_host_mirror(cuda, kind):
     n = int(w[0])
     assert n == len(host)
     header = (4 + len(b.q_lens) + 1 + 3) // 4 * 4
-    items = w[header:header + 4 * n].reshape(n, 4)
-    assert (items[:, 3] == 0).all()
-    dev = items[:, :3]
+    dev = w[header:header + 4 * n].reshape(n, 4)
     assert (np.diff(dev[:, 2]) <= 0).all()
     as_set = lambda a: sorted(map(tuple, a.tolist()))
     assert as_set(dev) == as_set(host)
@@ -234,10 +232,15 @@ def test_config3_shared_kv_tasks_sampled_rows(cuda):
         assert_identity(task_sums(v, dv, whole_k, 8), task_sums(out, do, whole_q, 8), "<V,dV> = <O,dO>")
 
 
-def test_ops_replay_from_a_captured_graph(cuda):
+@pytest.mark.parametrize("deterministic", [True, False])
+def test_ops_replay_from_a_captured_graph(cuda, deterministic):
     """Every entry point only enqueues work on the caller's stream (no allocation, no host
     synchronisation), so a tick can be captured once and replayed.  The replays run with other
-    eager work in between and with changed inputs, and must match eager results each time."""
+    eager work in between and with changed inputs, and must match eager results each time: bit for
+    bit, except dk and dv of the non-deterministic backward, which on a batch this small cuts key
+    blocks into pieces and adds their sums with float atomics in whatever order they finish (the
+    fp32 accumulators they go through are cleared by a kernel of the tick, so the replays test that
+    too)."""
     from distca_amd import workloads
     from distca_amd._lib import CaParams, load
     from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
@@ -261,7 +264,7 @@ def test_ops_replay_from_a_captured_graph(cuda):
     def tick():
         o, l = ca_varlen_fwd(q, k, v, cu, cu, 700, 700, workspace=ws)
         out.copy_(o); lse.copy_(l)
-        ca_varlen_bwd(do, q, k, v, out, lse, cu, cu, 700, 700, dq=dq, dk=dk, dv=dv, workspace=ws)
+        ca_varlen_bwd(do, q, k, v, out, lse, cu, cu, 700, 700, deterministic=deterministic, dq=dq, dk=dk, dv=dv, workspace=ws)
         a2a_memcpy_non_cp(dq.reshape(T, -1), off, shard, True, buffer=buf)
 
     side = torch.cuda.Stream()
@@ -281,7 +284,12 @@ def test_ops_replay_from_a_captured_graph(cuda):
         tick()                                                        # the same tick, eagerly
         torch.cuda.synchronize()
         for name, a_, b_ in zip(("out", "lse", "dq", "dk", "dv", "buf"), got, (out, lse, dq, dk, dv, buf)):
-            assert torch.equal(a_, b_), f"replay {rep}: {name} differs from the eager result"
+            if name in ("dk", "dv") and not deterministic:
+                # two orders of fp32 additions, each result rounded to bf16 once: a unit in the last place apart at most
+                err = (a_.float() - b_.float()).abs() / b_.float().abs().clamp_min(2.0 ** -6)
+                assert err.max().item() <= 2.0 ** -7, f"replay {rep}: {name} differs from the eager result by {err.max().item():.2e}"
+            else:
+                assert torch.equal(a_, b_), f"replay {rep}: {name} differs from the eager result"
 
 
 def test_server_ticks_in_place_equal_step_by_step_at_full_size(cuda):

@@ -36,8 +36,8 @@ def test_forward_items_tile_each_task_once_and_cover_visible_keys(lq, lk, causal
     rows, kv = scheduler.tile_shape(scheduler.FWD, HQ, HKV)
     items = scheduler.build_schedule(scheduler.FWD, _cu(lq), _cu(lk), HQ, HKV, causal=causal)
     seen = {}
-    for t, b, c in items.tolist():
-        assert (t, b) not in seen
+    for t, b, c, w in items.tolist():
+        assert (t, b) not in seen and w == 1 << 16          # forward items are never cut
         seen[(t, b)] = c
     for t, (a, k) in enumerate(zip(lq, lk)):
         nblk = -(-a * G // rows)
@@ -55,8 +55,21 @@ def test_forward_items_tile_each_task_once_and_cover_visible_keys(lq, lk, causal
 def test_backward_items_cover_every_query_block_that_sees_the_key_block(lq, lk, causal):
     rows, kv = scheduler.tile_shape(scheduler.BWD, HQ, HKV)
     items = scheduler.build_schedule(scheduler.BWD, _cu(lq), _cu(lk), HQ, HKV, causal=causal)
-    seen = {(t, b): c for t, b, c in items.tolist()}
-    assert len(seen) == len(items)
+    whole = scheduler.whole_items(items)
+    seen = {(t, b): c for t, b, c in whole.tolist()}
+    assert len(seen) == len(whole)
+    # these batches are small, so expensive key blocks come in pieces: piece j of k, each once, of
+    # consecutive query blocks counted from the last block down (cost n: blocks [n j / k, n (j+1) / k))
+    pieces = {}
+    for t, b, c, w in items.tolist():
+        pieces.setdefault((t, b), []).append((w & 0xffff, w >> 16, c))
+    for (t, b), ps in pieces.items():
+        k = ps[0][1]
+        assert sorted(j for j, _, _ in ps) == list(range(k)) and all(kk == k for _, kk, _ in ps)
+        n = seen[(t, b)]
+        assert all(c == n * (j + 1) // k - n * j // k for j, _, c in ps)
+    det = scheduler.build_schedule(scheduler.BWD, _cu(lq), _cu(lk), HQ, HKV, causal=causal, deterministic=True)
+    assert (det[:, 3] == 1 << 16).all() and sorted(map(tuple, det[:, :3].tolist())) == sorted(map(tuple, whole.tolist()))
     for t, (a, k) in enumerate(zip(lq, lk)):
         nkb = -(-k // kv) if a > 0 else 0
         assert sorted(b for (tt, b) in seen if tt == t) == list(range(nkb))
@@ -109,7 +122,7 @@ def test_sorted_dispatch_balances_a_skewed_batch(kind):
 
 
 def test_empty_batch_and_empty_tasks():
-    assert scheduler.build_schedule(scheduler.FWD, [0], [0], HQ, HKV).shape == (0, 3)
+    assert scheduler.build_schedule(scheduler.FWD, [0], [0], HQ, HKV).shape == (0, 4)
     items = scheduler.build_schedule(scheduler.FWD, _cu([0, 0, 4]), _cu([9, 0, 4]), HQ, HKV)
     assert set(items[:, 0].tolist()) == {2}
     items = scheduler.build_schedule(scheduler.BWD, _cu([0, 4]), _cu([700, 4]), HQ, HKV)
