@@ -948,7 +948,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     const int64_t max_items = bwd_max_items(p);
     rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_kv), max_items, s);
     if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
+    const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_kv);
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
@@ -965,7 +965,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     const int64_t max_items = dq_max_items(p);
     rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
     if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
+    const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_q);
     a.zero_row = ws + w.sched_q + sched_zero_row_off(p->num_tasks, max_items);

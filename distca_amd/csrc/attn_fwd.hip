@@ -481,7 +481,7 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   a.q_task_off = q_task_off; a.out_task_off = out_task_off; a.q_tok_bytes = q_tok_bytes; a.out_tok_bytes = out_tok_bytes;
   a.lse_in_token = lse ? 0 : 1;
-  const int64_t grid = max_items * p->num_heads_kv * kSchedOversub;
+  const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
   if (first_use_on_this_device(kSlotFwdLds)) {
     hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);

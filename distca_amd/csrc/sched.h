@@ -107,7 +107,8 @@ DISTCA_HD int64_t sched_zero_row_off(int32_t num_tasks, int64_t max_items) {
   return (sched_bytes(num_tasks, max_items) + 255) / 256 * 256;
 }
 // After the zero row: one ticket counter per kv head, zeroed by the builder.  The attention kernels
-// are launched with kSchedOversub workgroups per (item, kv head).  A workgroup does not work on the
+// are launched with 5/4 workgroups per (item, kv head) -- the surplus is what a fast XCD takes over from
+// a slow one; the XCDs of a device were seen up to 8 % apart -- and a workgroup does not work on the
 // item its id names: it draws the next ticket of its home head (id % Hkv), which is the rank of its
 // item in the sorted list, and when that head's list is used up it draws from the other heads; it
 // exits when all are used up.  Workgroup ids are dealt round-robin over the XCDs, and the XCDs of one
@@ -116,7 +117,7 @@ DISTCA_HD int64_t sched_zero_row_off(int32_t num_tasks, int64_t max_items) {
 // whereas now an XCD that finishes its own heads early takes items of the others.
 constexpr int64_t kTicketBytes = 1024;
 constexpr int32_t kSchedMaxHeads = (int32_t)(kTicketBytes / 4);
-constexpr int32_t kSchedOversub = 2;
+constexpr int32_t kSchedOversubNum = 5, kSchedOversubDen = 4;
 DISTCA_HD int64_t sched_ticket_off(int32_t num_tasks, int64_t max_items) {
   return sched_zero_row_off(num_tasks, max_items) + kZeroRowBytes;
 }
@@ -128,19 +129,35 @@ DISTCA_HD int64_t sched_region_bytes(int32_t num_tasks, int64_t max_items) {
 // Draws this workgroup's (item rank, kv head); false when every list is used up.  `slot` is two ints
 // of LDS that the caller may reuse afterwards.  All threads of the workgroup must call it.
 __device__ __forceinline__ bool take_item(int32_t *tickets, int32_t nitems, int32_t hkv, int32_t *slot, int &item, int &kvh) {
-  if (threadIdx.x == 0) {
-    int q = (int)(blockIdx.x % (unsigned)hkv), t = -1;
-    for (int d = 0; d < hkv; ++d) {
-      // counters only grow: a list seen as used up stays so, and a stale smaller value only costs the atomic
-      if (__builtin_nontemporal_load(tickets + q) < nitems) {
-        t = atomicAdd(tickets + q, 1);
-        if (t < nitems) break;
-        t = -1;
+  if (threadIdx.x < 64) {  // the first wave
+    // One look at all the counters at once (a lane per head): a workgroup that comes when every list is used
+    // up -- half of the launch's workgroups -- leaves after a single round trip to memory.  Counters only
+    // grow: a list seen as used up stays so, and a stale smaller value only costs an atomic.
+    const int lane = threadIdx.x;
+    const int home = (int)(blockIdx.x % (unsigned)hkv);
+    int t = -1, q = home;
+    for (int base = 0; base < hkv && t < 0; base += 64) {
+      int h = home + base + lane;
+      while (h >= hkv) h -= hkv;
+      const bool live = base + lane < hkv && __builtin_nontemporal_load(tickets + h) < nitems;
+      unsigned long long avail = __ballot(live);
+      // heads in the order home, home + 1, ...: lane d of this round looked at head home + base + d
+      while (avail && t < 0) {
+        const int d = __builtin_ctzll(avail);
+        avail &= avail - 1;
+        q = home + base + d;
+        while (q >= hkv) q -= hkv;
+        if (lane == 0) {
+          t = atomicAdd(tickets + q, 1);
+          if (t >= nitems) t = -1;
+        }
+        t = __shfl(t, 0, 64);
       }
-      if (++q == hkv) q = 0;
     }
-    slot[0] = t;
-    slot[1] = q;
+    if (lane == 0) {
+      slot[0] = t;
+      slot[1] = q;
+    }
   }
   __syncthreads();
   item = __builtin_amdgcn_readfirstlane(slot[0]);
