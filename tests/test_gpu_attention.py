@@ -56,10 +56,10 @@ def test_whole_docs_fwd_bwd_medium(cuda):
     _run([512, 1024, 700], [512, 1024, 700], 32, 8, 2, cuda)
 
 
-@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 1), (6, 2), (16, 2), (64, 1), (24, 8), (32, 1), (16, 16), (3, 3)])
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 1), (6, 2), (16, 2), (64, 1), (24, 8), (32, 1), (16, 16), (3, 3), (80, 80)])
 def test_head_groupings(cuda, hq, hkv):
-    """MHA (also with 16 and with 3 kv heads: more lists of work items than XCDs, and a count that does not divide
-    their number), MQA, a non-power-of-two group, the Llama-3-70B group of 8; groups of 64 (more heads per token than a
+    """MHA (also with 16, 3 and 80 kv heads: more lists of work items than XCDs, a count that does not divide
+    their number, and more lists than a wave has lanes to look at them), MQA, a non-power-of-two group, the Llama-3-70B group of 8; groups of 64 (more heads per token than a
     backward row block holds), of 3 (a row block does not start at a token boundary) and of 32 (exactly one)."""
     # dK and dV of a kv head sum the bf16-rounded P and dS of all its query heads: with 32 or 64 of them the
     # rounding noise of the sum (growing as the square root of the count) is allowed twice the bar
