@@ -80,6 +80,27 @@ def test_non_causal(cuda):
     _run([100, 260], [100, 260], 4, 2, 6, cuda, causal=False)
 
 
+def test_long_document_in_pieces(cuda):
+    """One document of 4096 tokens: too few key blocks to occupy the device, so the backward cuts every key
+    block into pieces of consecutive query blocks (the first block into about thirty) and adds their dK/dV in
+    fp32; also a deterministic run of the same, whole blocks, bit for bit equal to a second one."""
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    _run([4096], [4096], 8, 2, 11, cuda)
+    q, k, v, do = (t.to(cuda) for t in make_qkv(4096, 4096, 8, 2, 128, 11))
+    c = torch.tensor(cu([4096]), device=cuda)
+    out, lse = ca_varlen_fwd(q, k, v, c, c, 4096, 4096, None, True, None)
+    a = ca_varlen_bwd(do, q, k, v, out, lse, c, c, 4096, 4096, None, True, True, None)
+    b = ca_varlen_bwd(do, q, k, v, out, lse, c, c, 4096, 4096, None, True, True, None)
+    torch.cuda.synchronize()
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    n = ca_varlen_bwd(do, q, k, v, out, lse, c, c, 4096, 4096, None, True, False, None)
+    torch.cuda.synchronize()
+    for x, y, name in zip(n, a, ("dq", "dk", "dv")):
+        # same products, summed per piece and then across pieces in fp32: a bf16 unit in the last place apart at most
+        err = ((x.float() - y.float()).abs() / y.float().abs().clamp_min(2.0 ** -6)).max().item()
+        assert err <= 2.0 ** -7, f"{name}: pieces against whole blocks {err:.2e}"
+
+
 def test_empty_task(cuda):
     _run([128, 0, 70], [128, 0, 70], 4, 2, 8, cuda)
 
