@@ -20,7 +20,7 @@
 //      that every SIMD holds two waves at different points of the loop body and a block is
 //      fetched once for 256 keys.  Per block and wave:
 //        S = Q K^T, dP = dO V^T            A from the query tile, B = K registers / V tile (LDS)
-//        P = exp2(S*c - lse2), dS = P (dP*scale - delta*scale)          in registers
+//        P = exp2(S*c - lse2), dS / scale = P (dP - delta)              in registers
 //        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
 //                                          B = the accumulator registers converted to bf16
 //      Query tiles arrive two periods ahead through LDS-direct global loads (each wave brings
@@ -72,7 +72,7 @@ static_assert(kBwdLds <= 160 * 1024, "LDS budget");
 
 struct BwdArgs {
   const __bf16 *q, *k, *v, *dout;
-  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and delta*scale
+  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and -delta
   __bf16 *dq, *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
@@ -261,11 +261,17 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
   auto phase_a = [&](int stage) {
     const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
+    // dP accumulates on top of -delta of its rows (register r of the accumulator is query row 8 (r / 4) + 4 g + r % 4),
+    // so that phase B has dP - delta without an instruction; the scale is applied to dK once, at the end
+    const uint8_t *stat_a = lds + kStatOff + stage * kStatBytes + kBM * 4;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      sacc[r] = 0.f;
-      dpacc[r] = 0.f;
+    for (int cq = 0; cq < 4; ++cq) {
+      const f32x4 nd = *reinterpret_cast<const f32x4 *>(stat_a + (8 * cq + 4 * g) * 4);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) dpacc[4 * cq + rr] = nd[rr];
     }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
     // operands of step s+1 are requested before the MFMAs of step s are issued
     constexpr int kDa = 2;  // operand fetch distance in MFMA steps
     bf16x8 qa[kDa], da[kDa], vb[kDa];
@@ -300,7 +306,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       for (int cq = 0; cq < 4; ++cq) {
         const int qr = 8 * cq + 4 * g;
         const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + qr * 4);
         i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
         if constexpr (decltype(masked)::value) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
 #pragma unroll
@@ -310,7 +315,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
           if constexpr (decltype(masked)::value) {
             if (kw0 + l32 > lim4[rr]) p = 0.f;
           }
-          const float ds = p * __builtin_fmaf(dpacc[r], a.scale, -del4[rr]);
+          const float ds = p * dpacc[r];
           sacc[r] = p;
           dpacc[r] = ds;
         }
@@ -413,6 +418,10 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   wait_vm0();  // nothing may still be on its way into LDS when the workgroup ends
 
   // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dkacc[db][r] *= a.scale;
   if (ALIAS) {
     // Work items that share K/V rows (tasks over one stored prefix, pieces of one key block) add up in
     // fp32; the order of these additions is the one source of run-to-run variation.  A lane holds one key's
@@ -516,7 +525,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     if (valid[m]) {
       const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
       lse2[m] = a.lse2[so];
-      dsc[m] = a.dscaled[so];
+      dsc[m] = -a.dscaled[so] * a.scale;
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -729,7 +738,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   }
 }
 
-// Per (token, head) row: dscaled[h][t] = scale * sum_d dO*O and lse2[h][t] = lse[h][t]*log2(e).
+// Per (token, head) row: dscaled[h][t] = -sum_d dO*O (minus delta, unscaled; the name is historical) and lse2[h][t] = lse[h][t]*log2(e).
 // dout and out point at their part of token 0 of a region laid out like BwdArgs' query side; lse is
 // [Hq][Tq] fp32, or, when lse_tok is given instead, Hq fp32 per token at lse_tok + token start.
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restrict__ dout, const uint8_t *__restrict__ out,
@@ -768,7 +777,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restr
   for (int o = 8; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
   if (row < rows && sub == 0) {
     const int64_t o = (int64_t)h * total_q + t;
-    dscaled[o] = s * scale;
+    dscaled[o] = -s;  // minus delta, unscaled: the start value of the dP accumulators in dkdv
     const float l = lse_tok ? reinterpret_cast<const float *>(lse_tok + tok_start)[h] : lse[o];
     lse2[o] = l * kLog2e;
   }
