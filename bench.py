@@ -35,7 +35,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
 # WRITE_SIZE (x1.000), factors from the pack kernel's known copy size in the same run
-MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.92e9, "ca_bwd_dkdv_kernel": 33.81e9, "ca_bwd_dq_kernel": 12.60e9}
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.92e9, "ca_bwd_dkdv_kernel": 35.18e9, "ca_bwd_dq_kernel": 12.72e9}
 
 
 def log(*a):
