@@ -957,7 +957,10 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     const int64_t max_items = bwd_max_items(p);
     rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_kv), max_items, s);
     if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
+    // the list is sized for tasks over shared K/V rows; without them the tighter bound sizes the grid (a batch of
+    // many short documents and one long one would otherwise launch mostly workgroups that find nothing to do)
+    const int64_t grid_items = alias ? max_items : bwd_key_blocks_own_rows(p) + bwd_split_target(p);
+    const int64_t grid = grid_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_kv);
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));

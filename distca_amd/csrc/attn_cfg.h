@@ -63,16 +63,18 @@ constexpr int kNumCUs = 256;
 // device twice over, unless the caller asked for a deterministic backward (the pieces' dK/dV are added up with
 // float atomics).  Returns the number of pieces to aim for per kv head, 0 = no cutting.
 constexpr int kSplitPiecesPerCU = 2;
+// Upper bounds, from host-known sizes, of the number of key blocks = sum over tasks of ceil(Lk / kBwdKV).
+// When every task has its own K/V rows the Lk add up to total_k at most; when tasks read shared rows
+// (kv_task_offsets) only Lk <= max_seqlen_k is known.
+inline int64_t bwd_key_blocks_own_rows(const distca_ca_params *p) { return (int64_t)p->total_k / kBwdKV + p->num_tasks + 1; }
 inline int64_t bwd_key_blocks_bound(const distca_ca_params *p) {
-  // sum over tasks of ceil(Lk / kBwdKV); sum of Lk may exceed total_k when prefixes alias,
-  // but each Lk <= max_seqlen_k.
-  const int64_t by_total = (int64_t)p->total_k / kBwdKV + p->num_tasks + 1;
+  const int64_t by_total = bwd_key_blocks_own_rows(p);
   const int64_t by_max = ((int64_t)p->max_seqlen_k / kBwdKV + 1) * p->num_tasks + 1;
   return by_total > by_max ? by_total : by_max;
 }
 inline int32_t bwd_split_target(const distca_ca_params *p) {
   if (p->deterministic) return 0;
-  if (bwd_key_blocks_bound(p) * p->num_heads_kv >= 2 * kNumCUs) return 0;
+  if (bwd_key_blocks_own_rows(p) * p->num_heads_kv >= 2 * kNumCUs) return 0;
   const int32_t t = kSplitPiecesPerCU * kNumCUs / p->num_heads_kv;
   return t > 0 ? t : 1;
 }
