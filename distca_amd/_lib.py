@@ -43,6 +43,7 @@ SYMBOLS = {
     "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_schedule_capacity": (c_int64, [c_int, POINTER(CaParams)]),
     "distca_ca_schedule_host": (c_int64, [c_int, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64]),
     "distca_timing_enable": (None, [c_int]),
     "distca_timing_read": (c_int, [c_int, POINTER(ctypes.c_double), POINTER(c_int64)]),

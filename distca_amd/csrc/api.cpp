@@ -24,11 +24,26 @@ int num_compute_units() {
   return cached[dev];
 }
 
-bool first_use_on_this_device(int slot) {
-  static std::atomic<unsigned char> seen[64][kSlotCount];
+namespace {
+std::atomic<unsigned char> &setup_flag(int slot, bool *ok) {
+  static std::atomic<unsigned char> done[64][kSlotCount];
+  static std::atomic<unsigned char> none;
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || slot < 0 || slot >= kSlotCount) return true;
-  return seen[dev][slot].exchange(1) == 0;
+  *ok = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && slot >= 0 && slot < kSlotCount;
+  return *ok ? done[dev][slot] : none;
+}
+}  // namespace
+
+bool device_setup_pending(int slot) {
+  bool ok;
+  std::atomic<unsigned char> &f = setup_flag(slot, &ok);
+  return !ok || f.load(std::memory_order_acquire) == 0;
+}
+
+void device_setup_done(int slot) {
+  bool ok;
+  std::atomic<unsigned char> &f = setup_flag(slot, &ok);
+  if (ok) f.store(1, std::memory_order_release);
 }
 
 namespace {

@@ -39,9 +39,12 @@ struct ScopedTimer {
 
 // Number of compute units of the current device (cached per device id).
 int num_compute_units();
-// True the first time it is called with `slot` on the current device: per-device set-up such as
-// raising a kernel's dynamic LDS limit is done once for each GPU the library runs on.
-bool first_use_on_this_device(int slot);
+// Per-device set-up such as raising a kernel's dynamic LDS limit is done once for each GPU the library runs
+// on: pending() is true until done() has been called for `slot` on the current device.  The flag is set only
+// after the set-up calls have succeeded, so a second host thread never launches ahead of them (two threads
+// may both do the set-up, which is idempotent).
+bool device_setup_pending(int slot);
+void device_setup_done(int slot);
 enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotCount = 2 };
 
 }  // namespace distca

@@ -752,9 +752,15 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restr
   float s = 0.f;
   int64_t t = 0, tok_start = 0;
   int h = 0;
-  if (row < rows) {
+  bool live = row < rows;
+  if (live) {
     t = row / hq;
     h = (int)(row - t * hq);
+    // tokens past the last task (total_q may exceed the tasks' rows) belong to no shard: nothing is read for them,
+    // and their statistics make P = exp2(s - inf) = 0 wherever a kernel might look
+    live = t < cu_q[num_tasks];
+  }
+  if (live) {
     if (task_off) {
       // the task that holds token t: last b with cu_q[b] <= t
       int lo = 0, hi = num_tasks - 1;
@@ -778,8 +784,34 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restr
   if (row < rows && sub == 0) {
     const int64_t o = (int64_t)h * total_q + t;
     dscaled[o] = -s;  // minus delta, unscaled: the start value of the dP accumulators in dkdv
-    const float l = lse_tok ? reinterpret_cast<const float *>(lse_tok + tok_start)[h] : lse[o];
+    float l = INFINITY;
+    if (live) l = lse_tok ? reinterpret_cast<const float *>(lse_tok + tok_start)[h] : lse[o];
     lse2[o] = l * kLog2e;
+  }
+}
+
+// Zeroes the dk / dv rows that no workgroup of the dK/dV kernel writes when every task owns its K/V rows: the
+// rows of tasks without queries (they get no work item) and the rows past the last task.  Workgroup (b, y):
+// part y of task b's rows, b == num_tasks standing for the tail.
+__global__ __launch_bounds__(256) void fill_unowned_rows_kernel(u32x4 *__restrict__ dk, u32x4 *__restrict__ dv,
+                                                               const int32_t *__restrict__ cu_q, const int32_t *__restrict__ cu_k,
+                                                               int32_t num_tasks, int32_t total_k, int64_t row_vecs) {
+  const int b = blockIdx.x;
+  int64_t r0, r1;
+  if (b < num_tasks) {
+    if (cu_q[b + 1] > cu_q[b]) return;
+    r0 = cu_k[b];
+    r1 = cu_k[b + 1];
+  } else {
+    r0 = cu_k[num_tasks];
+    r1 = total_k;
+  }
+  if (r0 < 0) r0 = 0;
+  if (r1 > total_k) r1 = total_k;
+  const int64_t v0 = r0 * row_vecs, v1 = r1 * row_vecs;
+  for (int64_t i = v0 + (int64_t)blockIdx.y * 256 + threadIdx.x; i < v1; i += (int64_t)gridDim.y * 256) {
+    dk[i] = u32x4{0, 0, 0, 0};
+    dv[i] = u32x4{0, 0, 0, 0};
   }
 }
 
@@ -917,9 +949,14 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     if (use_acc) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 2)), dim3(256), 0, s, (u32x4 *)(ws + w.dk_acc),
                          (w.total - w.dk_acc) / 16);
-    } else {
+    } else if (p->num_tasks == 0 || p->total_q == 0) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dk, kv_elems / 8);
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dv, kv_elems / 8);
+    } else {
+      // every task owns its rows and the dK/dV kernel writes each row of a task that has queries exactly once:
+      // only the others need the fill (at 131 072 tokens that is 0.5 GB of writes not made)
+      hipLaunchKernelGGL(fill_unowned_rows_kernel, dim3((unsigned)p->num_tasks + 1, 16), dim3(256), 0, s, (u32x4 *)dk, (u32x4 *)dv,
+                         cu_q, cu_k, p->num_tasks, p->total_k, (int64_t)p->num_heads_kv * kHeadDim / 8);
     }
   }
   if (p->num_tasks == 0 || p->total_q == 0) return check_launch("ca_bwd(clear)");
@@ -944,11 +981,12 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
   if ((uint64_t)p->max_seqlen_q * a.group * a.group >= (1ull << 32))
     return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: max_seqlen_q * (Hq/Hkv)^2 must stay below 2^32");
 
-  if (first_use_on_this_device(kSlotBwdLds)) {
+  if (device_setup_pending(kSlotBwdLds)) {
     hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
     hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
     hipError_t e3 = hipFuncSetAttribute((const void *)ca_bwd_dq_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
     if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve LDS");
+    device_setup_done(kSlotBwdLds);
   }
 
   // ---- dK, dV: one workgroup per (task, 256-key block, kv head)

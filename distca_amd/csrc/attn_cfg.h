@@ -57,8 +57,6 @@ inline SchedGeom fwd_geom(const distca_ca_params *p) {
   g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_k / kFwdKV + 1);
   return g;
 }
-// Compute units of the device this library is built for (MI355X).
-constexpr int kNumCUs = 256;
 // Key blocks are cut into pieces (sched.h) when the batch has so few of them that they could not occupy the
 // device twice over, unless the caller asked for a deterministic backward (the pieces' dK/dV are added up with
 // float atomics).  Returns the number of pieces to aim for per kv head, 0 = no cutting.
@@ -74,8 +72,9 @@ inline int64_t bwd_key_blocks_bound(const distca_ca_params *p) {
 }
 inline int32_t bwd_split_target(const distca_ca_params *p) {
   if (p->deterministic) return 0;
-  if (bwd_key_blocks_own_rows(p) * p->num_heads_kv >= 2 * kNumCUs) return 0;
-  const int32_t t = kSplitPiecesPerCU * kNumCUs / p->num_heads_kv;
+  const int cus = num_compute_units();  // of the current device; 256 when there is none (the host mirror on a CPU box)
+  if (bwd_key_blocks_own_rows(p) * p->num_heads_kv >= 2 * cus) return 0;
+  const int32_t t = kSplitPiecesPerCU * cus / p->num_heads_kv;
   return t > 0 ? t : 1;
 }
 inline SchedGeom dq_geom(const distca_ca_params *p) {
@@ -103,7 +102,7 @@ inline int64_t dq_max_items(const distca_ca_params *p) {
   return (int64_t)p->total_q * group / kDqRows + p->num_tasks + 1;
 }
 inline int64_t bwd_max_items(const distca_ca_params *p) {
-  // cutting adds at most total cost / piece <= split_target pieces to the key blocks
+  // cutting adds at most total cost / piece <= split_target pieces to the key blocks (piece_size rounds up)
   return bwd_key_blocks_bound(p) + bwd_split_target(p);
 }
 

@@ -483,9 +483,10 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   a.lse_in_token = lse ? 0 : 1;
   const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
-  if (first_use_on_this_device(kSlotFwdLds)) {
+  if (device_setup_pending(kSlotFwdLds)) {
     hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
     if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
+    device_setup_done(kSlotFwdLds);
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);

@@ -117,6 +117,7 @@ __global__ __launch_bounds__(kPackThreads) void pack_kernel(
     total = c.total;
     if (total <= 0) return;
     cp = t0 / total;
+    if (cp >= max_cp) return;  // a tensor with more rows than the shards add up to: the slices past the last replica own nothing
     pos = t0 - cp * total;
     __syncthreads();
   }

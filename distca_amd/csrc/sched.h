@@ -34,10 +34,19 @@ struct SchedGeom {
 // Cutting key blocks: a batch of few tokens has fewer key blocks than the device has compute units, and
 // the block at the start of a long document streams every query row below it, so without cuts the launch
 // lasts as long as that one workgroup.  A block of cost c (query blocks to stream) is cut into
-// ceil(c / piece) pieces of consecutive query blocks, piece = max(kMinPiece, total cost / split_target);
+// ceil(c / piece) pieces of consecutive query blocks, piece = max(kMinPiece, ceil(total cost / split_target));
 // the pieces are independent work items whose dK/dV are added up in fp32.
 constexpr int32_t kMinPiece = 16;
 constexpr int32_t kMaxPieces = 64;
+// Piece size for a batch of `total_cost` query-block visits: the ceiling of total / target, so that the pieces
+// of all blocks together number at most target + (number of blocks) -- the bound the work list is sized by
+// (sum of ceil(c / piece) <= total / piece + blocks, and total / piece <= target only when piece is rounded up).
+DISTCA_HD int32_t piece_size(unsigned long long total_cost, int32_t split_target) {
+  if (split_target <= 0) return 0;
+  const unsigned long long per = (total_cost + (unsigned long long)split_target - 1) / (unsigned long long)split_target;
+  if (per <= (unsigned long long)kMinPiece) return kMinPiece;
+  return per < 0x7fffffffull ? (int32_t)per : 0x7fffffff;
+}
 DISTCA_HD int32_t piece_count(int32_t cost, int32_t piece) {
   if (piece <= 0) return 1;
   int32_t k = (cost + piece - 1) / piece;
@@ -93,7 +102,8 @@ inline int32_t pick_cost_shift(int64_t max_cost) {
 }
 
 // Workspace layout of a schedule (all int32):
-//   [0] item count   [1..3] reserved   [4 .. 4+B] exclusive block prefix per task
+//   [0] item count   [1] blocks   [2] entries dropped for lack of room (0 unless the caller's sizes understate
+//   its sequence lengths)   [3] reserved   [4 .. 4+B] exclusive block prefix per task
 //   then items as (task, block, cost, piece | pieces << 16) quadruples, 16-byte aligned.
 DISTCA_HD int64_t sched_header_ints(int32_t num_tasks) { return ((int64_t)4 + num_tasks + 1 + 3) / 4 * 4; }
 DISTCA_HD int64_t sched_bytes(int32_t num_tasks, int64_t max_items) {

@@ -88,8 +88,7 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
     }
     atomicAdd(&total_cost, local);
     __syncthreads();
-    const unsigned long long per = total_cost / (unsigned long long)g.split_target;
-    piece = per > (unsigned long long)kMinPiece ? (int32_t)(per < 0x7fffffffull ? per : 0x7fffffffull) : kMinPiece;
+    piece = piece_size(total_cost, g.split_target);
   }
 
   // 2. histogram of cost bins
@@ -142,6 +141,9 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
     const int32_t total = bins[0];
     ws[0] = total < max_items ? total : max_items;
     ws[1] = running;
+    // entries that found no room in the list (blocks beyond max_items count whole): never 0 < by construction
+    // when the caller's sizes bound its sequence lengths; tests and debugging read it
+    ws[2] = (total > max_items ? total - max_items : 0) + (running > max_items ? running - max_items : 0);
   }
   if (tid < kZeroRowBytes / 4) ws[sched_zero_row_off(num_tasks, max_items) / 4 + tid] = 0;
   if (tid < kTicketBytes / 4) ws[sched_ticket_off(num_tasks, max_items) / 4 + tid] = 0;
@@ -175,6 +177,16 @@ extern "C" int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t
   return DISTCA_OK;
 }
 
+extern "C" int64_t distca_ca_schedule_capacity(int kind, const distca_ca_params *p) {
+  if (!p) return fail(DISTCA_E_INVALID, "schedule_capacity: null params");
+  int rc = validate_params(p);
+  if (rc) return rc;
+  if (kind == 0) return fwd_max_items(p);
+  if (kind == 1) return bwd_max_items(p);
+  if (kind == 2) return dq_max_items(p);
+  return fail(DISTCA_E_INVALID, "schedule_capacity: kind must be 0 (fwd), 1 (bwd dK/dV) or 2 (bwd dQ)");
+}
+
 extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const int32_t *cu_k, const distca_ca_params *p,
                                            int32_t *items, int64_t max_items) {
   if (!p || !cu_q || !cu_k || (!items && max_items > 0)) return fail(DISTCA_E_INVALID, "schedule_host: null pointer");
@@ -196,8 +208,7 @@ extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const 
   }
   int32_t piece = 0;
   if (kind == 1 && g.split_target > 0) {
-    const unsigned long long per = total_cost / (unsigned long long)g.split_target;
-    piece = per > (unsigned long long)kMinPiece ? (int32_t)(per < 0x7fffffffull ? per : 0x7fffffffull) : kMinPiece;
+    piece = piece_size(total_cost, g.split_target);
   }
   for (const It &w : whole) {
     const int32_t k = piece_count(w.cost, piece);

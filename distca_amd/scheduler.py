@@ -34,14 +34,35 @@ def tile_shape(kind: int, hq: int, hkv: int, d: int = 128) -> Tuple[int, int]:
     return int(out[0]), int(out[1])
 
 
+DQ = 2  # a third list kind for capacity queries: the dQ kernel's blocks of query rows
+
+
+def schedule_capacity(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequence[int], num_heads_q: int,
+                      num_heads_kv: int, head_dim: int = 128, causal: bool = True, deterministic: bool = False,
+                      total_k: int | None = None) -> int:
+    """Room, in items, of the work list an attention call reserves in its workspace for this batch (sized on
+    the host from total_q, total_k, max_seqlen_* and the task count alone).  `total_k` overrides the sum of the
+    key lengths: tasks that share stored K/V rows (kv_task_offsets) have fewer rows than their lengths add up to."""
+    p = _params(cu_seqlens_q, cu_seqlens_k, num_heads_q, num_heads_kv, head_dim, causal, deterministic)
+    if total_k is not None:
+        p.total_k = int(total_k)
+    n = _lib.load().distca_ca_schedule_capacity(kind, ctypes.byref(p))
+    if n < 0:
+        _lib.check(int(n), "schedule_capacity")
+    return int(n)
+
+
 def build_schedule(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequence[int], num_heads_q: int,
-                   num_heads_kv: int, head_dim: int = 128, causal: bool = True, deterministic: bool = False) -> np.ndarray:
+                   num_heads_kv: int, head_dim: int = 128, causal: bool = True, deterministic: bool = False,
+                   total_k: int | None = None) -> np.ndarray:
     """Work items as an int32 array [n, 4] of (task, block, cost, piece | pieces << 16), most expensive
     first.  Backward items of a batch too small to occupy the device are cut into pieces of
     consecutive query blocks unless `deterministic`; everything else has pieces = 1, piece = 0."""
     cu_q = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
     cu_k = np.ascontiguousarray(cu_seqlens_k, dtype=np.int32)
     p = _params(cu_q, cu_k, num_heads_q, num_heads_kv, head_dim, causal, deterministic)
+    if total_k is not None:
+        p.total_k = int(total_k)
     lib = _lib.load()
     n = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), None, 0)
     if n < 0:

@@ -55,7 +55,10 @@ int distca_abi_version(void);
  * copy_seq_mask (int8 [num_seq], may be NULL) skips shards whose entry is 0;
  * like the reference it is honoured only when packing.
  * Rows at or beyond num_tokens are never touched.
- * token_bytes, seq_offset[] and both base pointers must be multiples of 16.
+ * token_bytes, seq_offset[] and both base pointers must be multiples of 16
+ * (token_bytes and the pointers are checked on the host; seq_offset[] and
+ * seq_tokens[] live on the device and are the caller's responsibility, as is
+ * sum(seq_tokens) >= num_tokens: rows past the last shard are left alone).
  * ------------------------------------------------------------------------- */
 int distca_memcpy_non_cp(void *tensor, void *buffer,
                          const int64_t *seq_offset, const int64_t *seq_tokens,
@@ -70,7 +73,12 @@ int distca_memcpy_non_cp(void *tensor, void *buffer,
  * seq_offset[c*num_seq + s].  Packing reads rows start_s.. of the
  * [num_tokens, token_bytes] tensor for every live replica c; unpacking writes
  * rows c*num_tokens + start_s.. of the [max_cp, num_tokens, token_bytes]
- * tensor (which the caller pre-zeroes, dispatch_fn.py:79-80). */
+ * tensor (which the caller pre-zeroes, dispatch_fn.py:79-80).
+ * seq_tokens must add up to num_tokens (the reference assumes the same,
+ * memcpy.cu:96-110); slices of a larger tensor that lie past the last replica
+ * are left alone.  seq_offset[] and seq_tokens[] are device arrays and are not
+ * checked: 16-byte alignment of the offsets and the ranges they name are the
+ * caller's responsibility, as in the reference. */
 int distca_memcpy_cp(void *tensor, void *buffer, const int8_t *do_shard,
                      const int64_t *seq_offset, const int64_t *seq_tokens,
                      int64_t token_bytes, int64_t num_tokens, int32_t max_cp,
@@ -95,6 +103,13 @@ int distca_grad_sum(void *data, int dtype, const int32_t *num_copies,
  * causal != 0 row i sees column j iff j <= i + (Lk - Lq) (bottom-right
  * aligned, the flash-attn 2.1+ convention the reference relies on at
  * per_doc_cp_attn.py:326,406-411).  q-head h reads kv-head h / (Hq/Hkv).
+ *
+ * The sizes in distca_ca_params must bound what the device arrays say, since the
+ * host sizes work lists and grids from them without reading device memory:
+ * cu_seqlens_q[B] <= total_q, every Lq <= max_seqlen_q, every Lk <= max_seqlen_k,
+ * and, when kv_task_offsets is NULL, cu_seqlens_k[B] <= total_k.  Work beyond
+ * those bounds is dropped (and counted, see distca_ca_schedule_capacity), never
+ * executed out of range.
  *
  * Layouts: q,out,dout,dq [total_q, Hq, D] bf16; k,v,dk,dv [total_k, Hkv, D]
  * bf16; lse [Hq, total_q] fp32 natural-log with the scale included;
@@ -205,6 +220,12 @@ int64_t distca_ca_schedule_host(int kind, const int32_t *cu_seqlens_q,
                                 const int32_t *cu_seqlens_k,
                                 const distca_ca_params *p, int32_t *items,
                                 int64_t max_items);
+/* Number of work items the list of `kind` (0 forward, 1 backward dK/dV, 2 backward dQ)
+ * has room for inside the workspace, computed from the sizes in p alone.  The device
+ * builder never writes more; it counts what did not fit in word 2 of the list's header
+ * (always 0 when p bounds the sequence lengths as required above).  No reference
+ * counterpart. */
+int64_t distca_ca_schedule_capacity(int kind, const distca_ca_params *p);
 /* tile geometry used by the kernels of `kind` for the head layout in p:
  * out[0] = query rows (tokens) per block, out[1] = kv rows per block. */
 int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);

@@ -189,6 +189,49 @@ def ca_reference_rows(
     return ob.permute(1, 0, 2), l.squeeze(-1), dqb
 
 
+def ca_reference_key_rows(
+    q_rows: torch.Tensor, dout_rows: torch.Tensor, out_rows: torch.Tensor, lse_rows: torch.Tensor,
+    k_rows: torch.Tensor, v_rows: torch.Tensor, row0: int, lq: int, lk: int, key0: int,
+    softmax_scale: Optional[float] = None, causal: bool = True, row_block: int = 16384,
+    dtype: torch.dtype = torch.float32,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dK, dV of a few keys of one task, for one kv head: the column view of ca_reference_bwd.
+
+    k_rows, v_rows [n, D]: keys key0 .. key0+n of the task (positions inside its prefix of lk keys).
+    q_rows, dout_rows, out_rows [R, G, D] and lse_rows [G, R]: query rows row0 .. row0+R of the task
+    (of its lq rows) for the G query heads of that kv head; the caller passes every row that sees one
+    of the keys (with the causal mask: rows >= key0 - (lk - lq)) -- rows it leaves out contribute
+    nothing to the result.  Gradients are formed from the saved forward results (out, lse) the way the
+    flash-attn backward invoked at fused_comm_attn.py:259-272 forms them:
+        P_ij = exp(s_ij - lse_i), D_i = <dO_i, out_i>, dS_ij = P_ij (<dO_i, v_j> - D_i),
+        dV_j = sum_{h, i} P_ij dO_i,  dK_j = scale sum_{h, i} dS_ij q_i.
+    Exists so that sampled dK/dV rows of tasks too long for the full fp32 evaluation can be checked."""
+    r, g, d = q_rows.shape
+    n = k_rows.shape[0]
+    scale = softmax_scale if softmax_scale is not None else d ** -0.5
+    kb = k_rows.to(dtype)
+    vb = v_rows.to(dtype)
+    dk = torch.zeros(n, d, dtype=dtype)
+    dv = torch.zeros(n, d, dtype=dtype)
+    j = torch.arange(key0, key0 + n).unsqueeze(0)
+    for a in range(0, r, row_block):
+        b = min(r, a + row_block)
+        qb = q_rows[a:b].to(dtype).permute(1, 0, 2)        # [G, R', D]
+        dob = dout_rows[a:b].to(dtype).permute(1, 0, 2)
+        ob = out_rows[a:b].to(dtype).permute(1, 0, 2)
+        l = lse_rows[:, a:b].to(dtype).unsqueeze(-1)       # [G, R', 1]
+        s = torch.matmul(qb, kb.t()) * scale               # [G, R', n]
+        if causal:
+            i = torch.arange(row0 + a, row0 + b).unsqueeze(1)
+            s = s.masked_fill((j > i + (lk - lq)).unsqueeze(0), float("-inf"))
+        p = torch.nan_to_num(torch.exp(s - l), nan=0.0)
+        delta = (dob * ob).sum(-1, keepdim=True)
+        ds = p * (torch.matmul(dob, vb.t()) - delta)
+        dv += torch.matmul(p.transpose(1, 2), dob).sum(0)
+        dk += torch.matmul(ds.transpose(1, 2), qb).sum(0) * scale
+    return dk, dv
+
+
 def causal_pairs(lq: int, lk: int, causal: bool = True) -> int:
     """Visible (query,key) pairs of one task: Lq*Lk - Lq(Lq-1)/2 under the bottom-right
     causal mask with Lk >= Lq — the work unit of Item.get_flops,

@@ -101,6 +101,38 @@ def test_long_document_in_pieces(cuda):
         assert err <= 2.0 ** -7, f"{name}: pieces against whole blocks {err:.2e}"
 
 
+@pytest.mark.parametrize("hq,hkv,n", [(128, 8, 989), (64, 8, 1345), (64, 8, 1364), (32, 8, 2999), (4, 1, 3000), (8, 2, 1500),
+                                      (16, 16, 7600), (16, 16, 7700)])
+def test_single_documents_around_the_piece_cutting_threshold(cuda, hq, hkv, n):
+    """One document per call, backward with key blocks cut into pieces: lengths at which the piece count comes
+    closest to the room the work list has (989 tokens at 128/8 heads and 1345 at 64/8 made one piece too many when
+    the piece size was rounded down), and a pair of lengths either side of the size from which blocks stay whole
+    (7680 tokens at 16 kv heads).  Gradients against the oracle, and the builder's count of entries it had no
+    room for must be zero."""
+    from distca_amd._lib import CaParams, load
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    import ctypes
+    q, k, v, do = make_qkv(n, n, hq, hkv, 128, 31)
+    c = cu([n])
+    dc = torch.tensor(c, device=cuda)
+    qd, kd, vd, dod = q.to(cuda), k.to(cuda), v.to(cuda), do.to(cuda)
+    p = CaParams(1, n, n, hq, hkv, 128, n, n, 128 ** -0.5, 1, 0, 0)
+    ws = torch.zeros(load().distca_ca_bwd_workspace_bytes(ctypes.byref(p)), dtype=torch.uint8, device=cuda)
+    print(f"case single document n={n} hq={hq} hkv={hkv}", flush=True)
+    out, lse = ca_varlen_fwd(qd, kd, vd, dc, dc, n, n)
+    dq, dk, dv = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dc, dc, n, n, None, True, False, None, workspace=ws)
+    torch.cuda.synchronize()
+    head = ws[:16].view(torch.int32).cpu()
+    assert int(head[2]) == 0, f"the key-block list dropped {int(head[2])} entries"
+    from distca_amd import scheduler
+    assert int(head[0]) == len(scheduler.build_schedule(scheduler.BWD, c, c, hq, hkv))
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, c, c, out=out.cpu(), softmax_lse=lse.cpu())
+    tol = dict(max_abs=4e-2, mean_rel=2e-3) if hq // hkv >= 16 else {}
+    assert_close_bf16(dq, ref_dq, "dq")
+    assert_close_bf16(dk, ref_dk, "dk", **tol)
+    assert_close_bf16(dv, ref_dv, "dv", **tol)
+
+
 def test_empty_task(cuda):
     _run([128, 0, 70], [128, 0, 70], 4, 2, 8, cuda)
 

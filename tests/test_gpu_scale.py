@@ -2,6 +2,8 @@
 full fp32 oracle (which would take hours on host cores at these sizes):
 
   * sampled query rows against the oracle (out, lse, dq for those rows over the whole prefix);
+  * sampled key rows against the oracle (dk, dv of those keys from every query row that sees them, summed
+    over the tasks that share the stored row);
   * <V, dV> = <O, dO>  (O is linear in V) and  <Q, dQ> = <K, dK>  (scores depend on Q K^T only,
     so scaling Q or K by 1+eps moves the loss equally), per kv head;
   * two runs give bit-identical results (no atomics anywhere in the unaliased path);
@@ -13,7 +15,7 @@ import pytest
 import torch
 
 from helpers import assert_close_bf16, assert_identity, randn_bf16, task_sums
-from oracle.attention import ca_reference_rows
+from oracle.attention import ca_reference_key_rows, ca_reference_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -73,6 +75,58 @@ def _check_sampled_rows(batch, q, k, v, do, out, lse, dq, rng, n_samples=6, rows
         assert_close_bf16(dq[sl], dq_ref, f"dq task {t}")
 
 
+def _rows_ref_group(batch, q, k, v, do, out, lse, t, r0, r1, kvh, g):
+    """Oracle (out, lse, dq) of rows [r0, r1) of task t for the g query heads of kv head kvh only: with 64 query
+    heads and a prefix of 262144 keys the full-width evaluation would hold 17 GB of repeated K/V on the host."""
+    q0 = int(batch.cu_seqlens_q[t])
+    lq, lk = int(batch.q_lens[t]), int(batch.k_lens[t])
+    k0 = int(batch.kv_task_offsets[t]) if batch.kv_task_offsets is not None else int(batch.cu_seqlens_k[t])
+    kvis = r1 + (lk - lq)                  # keys beyond the last sampled row's horizon are masked anyway
+    hs = slice(kvh * g, (kvh + 1) * g)
+    return ca_reference_rows(q[q0:q0 + r1, hs].cpu(), k[k0:k0 + kvis, kvh:kvh + 1].cpu(), v[k0:k0 + kvis, kvh:kvh + 1].cpu(),
+                             do[q0:q0 + r1, hs].cpu(), [0, r1], [0, kvis], 0, r0, r1,
+                             out_rows=out[q0 + r0:q0 + r1, hs].cpu(), lse_rows=lse[hs, q0 + r0:q0 + r1].cpu())
+
+
+def _check_rows_of_group(batch, q, k, v, do, out, lse, dq, t, r0, r1, kvh, g):
+    o_ref, l_ref, dq_ref = _rows_ref_group(batch, q, k, v, do, out, lse, t, r0, r1, kvh, g)
+    q0 = int(batch.cu_seqlens_q[t])
+    sl, hs = slice(q0 + r0, q0 + r1), slice(kvh * g, (kvh + 1) * g)
+    print(f"  rows task={t} [{r0},{r1}) of {int(batch.q_lens[t])}, prefix {int(batch.k_lens[t])}, kv head {kvh}", flush=True)
+    assert_close_bf16(out[sl, hs], o_ref, f"out task {t}")
+    assert (lse[hs, sl].cpu() - l_ref).abs().max().item() <= 2e-3
+    assert_close_bf16(dq[sl, hs], dq_ref, f"dq task {t}")
+
+
+def _check_key_rows(batch, q, k, v, do, out, lse, dk, dv, row0, n, kvh, g):
+    """dk, dv of stored K/V rows [row0, row0 + n) of kv head kvh against the oracle: the sum, over every task whose
+    prefix holds the rows, of the contributions of that task's query rows that see them."""
+    d = q.shape[2]
+    ref_k, ref_v = torch.zeros(n, d), torch.zeros(n, d)
+    hs = slice(kvh * g, (kvh + 1) * g)
+    used = []
+    for t in range(len(batch.q_lens)):
+        lq, lk = int(batch.q_lens[t]), int(batch.k_lens[t])
+        k0 = int(batch.kv_task_offsets[t]) if batch.kv_task_offsets is not None else int(batch.cu_seqlens_k[t])
+        lo, hi = max(row0, k0), min(row0 + n, k0 + lk)          # stored rows of the sample inside this task's prefix
+        if lo >= hi or lq == 0:
+            continue
+        j0 = lo - k0
+        first = max(0, j0 - (lk - lq))                           # rows before it see none of the keys
+        if first >= lq:
+            continue
+        q0 = int(batch.cu_seqlens_q[t])
+        rows = slice(q0 + first, q0 + lq)
+        gk, gv = ca_reference_key_rows(q[rows, hs].cpu(), do[rows, hs].cpu(), out[rows, hs].cpu(), lse[hs, rows].cpu(),
+                                       k[lo:hi, kvh].cpu(), v[lo:hi, kvh].cpu(), first, lq, lk, j0)
+        ref_k[lo - row0:hi - row0] += gk
+        ref_v[lo - row0:hi - row0] += gv
+        used.append((t, lq - first))
+    print(f"  keys stored rows [{row0},{row0 + n}) kv head {kvh}: (task, query rows) {used}", flush=True)
+    assert_close_bf16(dk[row0:row0 + n, kvh], ref_k, f"dk rows {row0}")
+    assert_close_bf16(dv[row0:row0 + n, kvh], ref_v, f"dv rows {row0}")
+
+
 def test_config2_llama8b_128k_properties(cuda):
     """The benchmark workload at full size: 131072 packed tokens, 32q/8kv heads."""
     from distca_amd import workloads
@@ -82,6 +136,13 @@ def test_config2_llama8b_128k_properties(cuda):
     for name, t in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
         assert torch.isfinite(t.float()).all(), name
     _check_sampled_rows(b, q, k, v, do, out, lse, dq, np.random.default_rng(0))
+    # dk / dv of sampled keys: the first, a middle and the last keys of the longest document, all keys of a short one
+    big = int(np.argmax(b.q_lens))
+    k_big, n_big = int(b.cu_seqlens_k[big]), int(b.k_lens[big])
+    small = int(np.argmin(b.q_lens))
+    for row0, n, kvh in ((k_big, 8, 0), (k_big + n_big // 2 + 77, 8, 5), (k_big + n_big - 8, 8, 7),
+                         (int(b.cu_seqlens_k[small]), 8, 3), (int(b.cu_seqlens_k[small]) + int(b.k_lens[small]) - 8, 8, 2)):
+        _check_key_rows(b, q, k, v, do, out, lse, dk, dv, row0, n, kvh, 4)
     # linearity identities per (task, kv head)
     cu = b.cu_seqlens_q
     assert_identity(task_sums(v, dv, cu, 8), task_sums(out, do, cu, 8), "<V,dV> = <O,dO>")
@@ -92,24 +153,69 @@ def test_config2_llama8b_128k_properties(cuda):
         assert torch.equal(x, y), f"{name} differs between two identical runs"
 
 
-def test_config5_llama70b_heads_forward_rows(cuda):
-    """64q/8kv heads (group 8) with one 262144-token document among short ones: forward at
-    full size, rows of the long document and of short ones against the oracle."""
+def test_config5_llama70b_heads_fwd_bwd_full_size(cuda):
+    """BASELINE config 5 as stated: 524288 packed tokens, one 262144-token document among lognormal ones, 64q/8kv heads,
+    forward and backward.  The backward at this size has 65536 query blocks per key block (the cost bins use a shift)
+    and a group of 8 heads per kv head.  Checked: sampled rows of out, lse, dq (the last rows of the long document
+    among them) and sampled key rows of dk, dv (first, middle, last keys of the long document; a short document)
+    against the oracle for one head group each, and the two linearity identities over every (task, kv head)."""
     from distca_amd import workloads
-    from distca_amd.fused_comm_attn import ca_varlen_fwd
     b = workloads.config5_llama70b_skewed()
-    q, k, v, do, cu_q, cu_k = _dev_inputs(b, 64, 8, cuda, 40)
-    print("cfg5 fwd", flush=True)
-    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, int(max(b.q_lens)), int(max(b.k_lens)))
-    torch.cuda.synchronize()
+    print("cfg5 fwd+bwd", flush=True)
+    q, k, v, do, out, lse, dq, dk, dv = _fwd_bwd(b, 64, 8, cuda, seed=40)
+    for name, t in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert torch.isfinite(t.float()).all(), name
     big = int(np.argmax(b.q_lens))
-    for t, r0 in ((big, int(b.q_lens[big]) - 8), (big, 100000), (0 if big else 1, 0)):
-        r1 = min(int(b.q_lens[t]), r0 + 8)
-        print(f"  rows task={t} [{r0},{r1})", flush=True)
-        o_ref, l_ref, _ = _rows_ref(b, q, k, v, None, t, r0, r1)
-        g0 = int(b.cu_seqlens_q[t]) + r0
-        assert_close_bf16(out[g0:g0 + r1 - r0], o_ref, f"out task {t}")
-        assert (lse[:, g0:g0 + r1 - r0].cpu() - l_ref).abs().max().item() <= 2e-3
+    n_big = int(b.q_lens[big])
+    short = 0 if big else 1
+    g = 8
+    for t, r0, kvh in ((big, n_big - 8, 6), (big, 100000, 1), (big, 0, 4), (short, max(0, int(b.q_lens[short]) - 8), 2)):
+        _check_rows_of_group(b, q, k, v, do, out, lse, dq, t, r0, min(int(b.q_lens[t]), r0 + 8), kvh, g)
+    k_big = int(b.cu_seqlens_k[big])
+    for row0, kvh in ((k_big, 3), (k_big + 100000, 1), (k_big + n_big - 8, 6), (int(b.cu_seqlens_k[short]), 2)):
+        _check_key_rows(b, q, k, v, do, out, lse, dk, dv, row0, 8, kvh, g)
+    cu = b.cu_seqlens_q
+    assert_identity(task_sums(v, dv, cu, 8), task_sums(out, do, cu, 8), "<V,dV> = <O,dO>")
+    assert_identity(task_sums(q, dq, cu, 8), task_sums(k, dk, cu, 8), "<Q,dQ> = <K,dK>")
+
+
+@pytest.mark.parametrize("variant", ["a", "b"])
+def test_config3_ca_tasks_full_size(cuda, variant):
+    """BASELINE config 3 at full size: 262144 query rows cut into CA tasks from 8 documents of up to 524288 tokens whose
+    K/V is stored once per document and read through kv_task_offsets (variant a: 64 tasks of 4096 rows; variant b:
+    chunks uniform in [4096, 32768]).  Sampled rows of out, lse, dq; sampled stored key rows of dk, dv, whose
+    reference is the sum over the tasks that read them; the linearity identities over the batch per kv head."""
+    from distca_amd import workloads
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    b = workloads.config3_ca_tasks(variant=variant)
+    q, k, v, do, cu_q, cu_k = _dev_inputs(b, 32, 8, cuda, 60)
+    kv_off = torch.tensor(b.kv_task_offsets, dtype=torch.int32, device=cuda)
+    mq, mk = int(max(b.q_lens)), int(max(b.k_lens))
+    print(f"cfg3{variant} full size: {len(b.q_lens)} tasks, {b.total_q} query rows, kv rows {b.kv_rows}, longest prefix {mk}", flush=True)
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+    dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+    torch.cuda.synchronize()
+    for name, t in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert torch.isfinite(t.float()).all(), name
+    rng = np.random.default_rng(2)
+    longest = int(np.argmax(b.k_lens))
+    tasks = [longest] + [int(t) for t in rng.choice(len(b.q_lens), size=3, replace=False)]
+    for i, t in enumerate(tasks):
+        lq = int(b.q_lens[t])
+        r0 = lq - 8 if i == 0 else int(rng.integers(0, lq - 8))
+        _check_rows_of_group(b, q, k, v, do, out, lse, dq, t, r0, r0 + 8, int(rng.integers(8)), 4)
+    # stored key rows: inside the query chunk of the task with the longest prefix (its diagonal), at the start of
+    # its document (read by every task of the document), and two more drawn from rows some task queries
+    k0, lk, lq = int(b.kv_task_offsets[longest]), int(b.k_lens[longest]), int(b.q_lens[longest])
+    samples = [(k0 + lk - lq + lq // 2, 1), (k0, 4), (k0 + lk - 8, 7)]
+    for t in tasks[1:3]:
+        kk, ll, qq = int(b.kv_task_offsets[t]), int(b.k_lens[t]), int(b.q_lens[t])
+        samples.append((kk + ll - qq + int(rng.integers(0, qq - 8)), int(rng.integers(8))))
+    for row0, kvh in samples:
+        _check_key_rows(b, q, k, v, do, out, lse, dk, dv, row0, 8, kvh, 4)
+    whole_q, whole_k = [0, b.total_q], [0, b.kv_rows]
+    assert_identity(task_sums(q, dq, whole_q, 8), task_sums(k, dk, whole_k, 8), "<Q,dQ> = <K,dK>")
+    assert_identity(task_sums(v, dv, whole_k, 8), task_sums(out, do, whole_q, 8), "<V,dV> = <O,dO>")
 
 
 def test_prefix_tasks_equal_whole_document(cuda):

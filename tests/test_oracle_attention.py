@@ -11,7 +11,7 @@ import torch.nn.functional as F
 import pytest
 
 from helpers import cu, make_qkv
-from oracle.attention import (attention_flops, ca_reference_bwd, ca_reference_fwd, ca_reference_rows, causal_pairs)
+from oracle.attention import (ca_reference_key_rows, attention_flops, ca_reference_bwd, ca_reference_fwd, ca_reference_rows, causal_pairs)
 
 
 def _rand(shape, seed, dtype=torch.float64):
@@ -188,6 +188,55 @@ def test_row_sampler_matches_full():
     dq, _, _ = ca_reference_bwd(do, q, k, v, cu(q_lens), cu(k_lens), dtype=torch.float64)
     o, l, g = ca_reference_rows(q, k, v, do, cu(q_lens), cu(k_lens), 0, 3, 9, dtype=torch.float64)
     assert torch.allclose(o, out[3:9]) and torch.allclose(l, lse[:, 3:9]) and torch.allclose(g, dq[3:9])
+
+
+def test_row_sampler_with_saved_forward_results_matches_full():
+    """The out_rows= / lse_rows= branch (what every full-size dq check on the GPU goes through) against
+    ca_reference_bwd(out=, softmax_lse=), itself pinned by autograd above when out and lse are exact.
+    The saved results are perturbed (bf16-rounded out, lse off by up to 1e-2) so that the branch is observably
+    different from recomputing them: the same rows without the saved results must NOT match."""
+    hq, hkv, d = 4, 2, 8
+    q_lens, k_lens = [11, 6], [20, 6]
+    q, k, v, do = _rand((17, hq, d), 25), _rand((26, hkv, d), 26), _rand((26, hkv, d), 27), _rand((17, hq, d), 28)
+    out, lse = ca_reference_fwd(q, k, v, cu(q_lens), cu(k_lens), dtype=torch.float64)
+    out_s = out.to(torch.bfloat16).double()
+    lse_s = lse + 1e-2 * torch.sin(torch.arange(lse.numel(), dtype=torch.float64)).reshape(lse.shape)
+    dq, _, _ = ca_reference_bwd(do, q, k, v, cu(q_lens), cu(k_lens), dtype=torch.float64, out=out_s, softmax_lse=lse_s)
+    for task, r0, r1, g0 in ((0, 3, 9, 3), (0, 0, 11, 0), (1, 2, 6, 13)):
+        _, _, g = ca_reference_rows(q, k, v, do, cu(q_lens), cu(k_lens), task, r0, r1, dtype=torch.float64,
+                                    out_rows=out_s[g0:g0 + r1 - r0], lse_rows=lse_s[:, g0:g0 + r1 - r0])
+        assert torch.allclose(g, dq[g0:g0 + r1 - r0], atol=1e-12)
+        _, _, g_plain = ca_reference_rows(q, k, v, do, cu(q_lens), cu(k_lens), task, r0, r1, dtype=torch.float64)
+        assert not torch.allclose(g_plain, dq[g0:g0 + r1 - r0], atol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_key_row_sampler_matches_full(causal):
+    """ca_reference_key_rows (dK/dV of a few keys of one task and kv head, from the query rows that see them)
+    against the same rows of ca_reference_bwd(out=, softmax_lse=), for a prefix task (lk > lq), for a whole
+    document, with perturbed saved results, with only the rows past the keys' horizon handed in, and in
+    several row blocks."""
+    hq, hkv, d = 6, 2, 8
+    g = hq // hkv
+    q_lens, k_lens = [11, 9], [20, 9]
+    cq, ck = cu(q_lens), cu(k_lens)
+    q, k, v, do = _rand((20, hq, d), 41), _rand((29, hkv, d), 42), _rand((29, hkv, d), 43), _rand((20, hq, d), 44)
+    out, lse = ca_reference_fwd(q, k, v, cq, ck, dtype=torch.float64, causal=causal)
+    out_s = out.to(torch.bfloat16).double()
+    lse_s = lse + 1e-2 * torch.cos(torch.arange(lse.numel(), dtype=torch.float64)).reshape(lse.shape)
+    _, dk, dv = ca_reference_bwd(do, q, k, v, cq, ck, dtype=torch.float64, out=out_s, softmax_lse=lse_s, causal=causal)
+    for task, key0, key1 in ((0, 0, 4), (0, 12, 17), (0, 17, 20), (1, 3, 9)):
+        lq, lk = q_lens[task], k_lens[task]
+        q0, k0 = int(cq[task]), int(ck[task])
+        first = max(0, key0 - (lk - lq)) if causal else 0          # rows before it see none of the keys
+        for kvh in range(hkv):
+            hs = slice(kvh * g, (kvh + 1) * g)
+            rows = slice(q0 + first, q0 + lq)
+            gk, gv = ca_reference_key_rows(q[rows, hs], do[rows, hs], out_s[rows, hs], lse_s[hs, rows],
+                                           k[k0 + key0:k0 + key1, kvh], v[k0 + key0:k0 + key1, kvh], first, lq, lk, key0,
+                                           causal=causal, row_block=4, dtype=torch.float64)
+            assert torch.allclose(gk, dk[k0 + key0:k0 + key1, kvh], atol=1e-12)
+            assert torch.allclose(gv, dv[k0 + key0:k0 + key1, kvh], atol=1e-12)
 
 
 def test_empty_rows_when_lk_lt_lq():

@@ -135,3 +135,49 @@ def test_group_sizes():
         items = scheduler.build_schedule(scheduler.FWD, _cu([100, 37]), _cu([100, 37]), hq, hkv)
         g = hq // hkv
         assert len(items) == -(-100 * g // rows) + -(-37 * g // rows)
+
+
+def _check_capacity_and_tiling(lq, lk, hq, hkv, total_k=None):
+    cu_q, cu_k = _cu(lq), _cu(lk)
+    items = scheduler.build_schedule(scheduler.BWD, cu_q, cu_k, hq, hkv, total_k=total_k)
+    cap = scheduler.schedule_capacity(scheduler.BWD, cu_q, cu_k, hq, hkv, total_k=total_k)
+    assert len(items) <= cap, f"lq={lq} lk={lk} heads {hq}/{hkv}: {len(items)} items for a list of {cap}"
+    return items
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (32, 8), (64, 8), (128, 8), (4, 1), (8, 2), (16, 4)])
+def test_backward_list_always_has_room_for_the_pieces(hq, hkv):
+    """The list is sized on the host as (bound on key blocks) + (pieces aimed for); the builder drops what does
+    not fit, so the piece size must be such that the count never exceeds it.  (With the piece size rounded down,
+    one document of 989 tokens at 128/8 heads, or of 1345 at 64/8, made one piece more than the list holds.)
+    Every document length up to the point where cutting stops, then a coarser sweep beyond."""
+    rows, kv = scheduler.tile_shape(scheduler.BWD, hq, hkv)
+    g = hq // hkv
+    lengths = list(range(1, 3000)) + list(range(3000, 16001, 37))
+    for n in lengths:
+        items = _check_capacity_and_tiling([n], [n], hq, hkv)
+        if n in (989, 1345, 1364, 2999) or n % 500 == 0:
+            # the pieces of every key block tile the query blocks that see it: [first block, nmb)
+            nmb = -(-n * g // rows)
+            got = {}
+            for t, b, c, w in items.tolist():
+                got.setdefault(b, []).append((w & 0xffff, w >> 16, c))
+            assert sorted(got) == list(range(-(-n // kv)))
+            for b, ps in got.items():
+                k = ps[0][1]
+                assert sorted(j for j, _, _ in ps) == list(range(k))
+                first = ((b * kv) * g) // rows
+                assert sum(c for _, _, c in ps) == nmb - first
+
+
+def test_backward_list_has_room_for_batches_and_shared_prefixes():
+    rng = np.random.default_rng(7)
+    for trial in range(300):
+        hq, hkv = [(32, 8), (64, 8), (8, 8), (4, 1), (128, 8)][trial % 5]
+        n = int(rng.integers(1, 9))
+        lq = rng.integers(0, 700, size=n)
+        extra = rng.integers(0, 900, size=n) * (rng.random(n) < 0.5)
+        lk = lq + extra
+        _check_capacity_and_tiling(lq.tolist(), lk.tolist(), hq, hkv)
+        # the same tasks over stored prefixes: fewer K/V rows than the lengths add up to
+        _check_capacity_and_tiling(lq.tolist(), lk.tolist(), hq, hkv, total_k=int(lk.max()))
