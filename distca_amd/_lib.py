@@ -38,6 +38,9 @@ SYMBOLS = {
     "distca_ca_bwd_workspace_bytes": (c_int64, [POINTER(CaParams)]),
     "distca_ca_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                               POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_fwd_noalloc_max_bytes": (c_int64, []),
+    "distca_ca_fwd_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      POINTER(CaParams), c_void_p]),
     "distca_ca_fwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                      c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),

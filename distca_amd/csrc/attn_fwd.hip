@@ -23,6 +23,8 @@
 // instruction, rows unpadded with swizzled 16-byte chunks, see tile_swz), one period ahead of
 // their use.
 #include <type_traits>
+#include <mutex>
+
 #include "api_util.h"
 #include "attn_cfg.h"
 #include "common.h"
@@ -418,6 +420,35 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
 
 using namespace distca;
 
+// Scratch memory of distca_ca_fwd_noalloc: the forward's work list, zero row and ticket counters, which every other
+// entry point takes from the caller's workspace.  One copy per GPU, held until the process ends.  The name below is
+// a host-side stand-in, never a device address: host code uses the per-device address from hipGetSymbolAddress.
+constexpr int64_t kNoAllocScratchBytes = 1 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+// Device address of `scratch` on the current device, resolved once per device with that device current.
+int noalloc_scratch(void **out) {
+  static std::mutex mu;
+  static void *ptr[64] = {nullptr};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= 64) return fail(DISTCA_E_UNSUPPORTED, "ca_fwd_noalloc: device id %d (at most 64 devices)", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(DISTCA_E_LAUNCH, "ca_fwd_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return DISTCA_OK;
+}
+}  // namespace
+
+extern "C" int64_t distca_ca_fwd_noalloc_max_bytes(void) { return kNoAllocScratchBytes; }
+
 extern "C" int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p) {
   if (!p) return fail(DISTCA_E_INVALID, "fwd_workspace_bytes: null params");
   int rc = validate_params(p);
@@ -439,6 +470,22 @@ extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *
   if (p->num_tasks == 0 || p->total_q == 0) return DISTCA_OK;
   if (!lse) return fail(DISTCA_E_INVALID, "ca_fwd: null pointer");
   return distca_ca_fwd_tokens(q, nullptr, 0, k, v, out, nullptr, 0, lse, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+}
+
+extern "C" int distca_ca_fwd_noalloc(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
+                                     const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_fwd_noalloc: null params");
+  const int64_t need = distca_ca_fwd_workspace_bytes(p);
+  if (need < 0) return (int)need;
+  if (need > kNoAllocScratchBytes)
+    return fail(DISTCA_E_WORKSPACE,
+                "ca_fwd_noalloc: this batch needs %lld B of scratch, the static array holds %lld B (about %lld work items: "
+                "query rows x heads per kv head / %d + tasks); use distca_ca_fwd with a workspace",
+                (long long)need, (long long)kNoAllocScratchBytes, (long long)(kNoAllocScratchBytes / 16), kFwdRows);
+  void *ws = nullptr;
+  const int rc = noalloc_scratch(&ws);
+  if (rc) return rc;
+  return distca_ca_fwd(q, k, v, out, lse, cu_q, cu_k, kv_off, p, ws, kNoAllocScratchBytes, stream);
 }
 
 extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,

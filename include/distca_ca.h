@@ -150,6 +150,26 @@ int distca_ca_fwd(const void *q, const void *k, const void *v, void *out,
                   const distca_ca_params *p, void *workspace,
                   int64_t workspace_bytes, void *stream);
 
+/* distca_ca_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot bring a
+ * workspace: the work list, zero row and ticket counters live in a static device array
+ * of distca_ca_fwd_noalloc_max_bytes() (1 MiB) inside the library, one copy per GPU,
+ * held until the process ends.  It has no counterpart in the reference (flash-attn
+ * allocates what it needs).  Same arguments, results and error codes as distca_ca_fwd
+ * without the workspace pair; a batch whose distca_ca_fwd_workspace_bytes exceeds the
+ * array is rejected with DISTCA_E_WORKSPACE (1 MiB holds about 65 000 work items, i.e.
+ * 16.7 million query rows x heads-per-kv-head: config 5 needs a quarter of it).  The call
+ * makes no hipMalloc / hipFree and rewrites everything it reads from the array, so it
+ * does not depend on what the previous call left there; every call on a GPU uses that
+ * GPU's one array, so calls that overlap on one GPU (two streams, two host threads)
+ * race and must be ordered by the caller. */
+int64_t distca_ca_fwd_noalloc_max_bytes(void);
+int distca_ca_fwd_noalloc(const void *q, const void *k, const void *v, void *out,
+                          float *lse, const int32_t *cu_seqlens_q,
+                          const int32_t *cu_seqlens_k,
+                          const int32_t *kv_task_offsets,
+                          const distca_ca_params *p, void *stream);
+
 /* The same forward with the query and output tokens where the CA server has them
  * (distca/runtime/megatron/ops/fused_comm_attn.py:298-389 unpacks q from the
  * receive buffer, runs attention, and packs [out | lse] tokens into the send
