@@ -76,14 +76,40 @@ def cpu_baseline(batch, budget_s: float, seed: int):
     }
 
 
+def _timed(torch, _lib, timer, fn, iters):
+    for _ in range(2):
+        fn()
+    torch.cuda.synchronize()
+    _lib.timing_read(timer)
+    _lib.timing_enable(True)
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    _lib.timing_enable(False)
+    ms, launches = _lib.timing_read(timer)
+    return ms / iters, launches // iters
+
+
+def _rate(bytes_moved, ms):
+    gbps = bytes_moved / (ms * 1e-3) / 1e9
+    return {"GB/s": round(gbps, 1), "frac_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4), "ms_per_pass": round(ms, 4)}
+
+
 def pack_unpack_bench(torch, dev, iters: int = 10):
-    """fa2a pack / unpack of 262 144 tokens of q (8 192 B) + k, v (2 048 B each): GB/s over
-    algorithmic bytes (read + write of the payload)."""
+    """The HBM-bound kernels of the path on 262 144 tokens, GB/s over algorithmic bytes (kernel durations by HIP events
+    on the launch stream):
+      pack / unpack   q (8 192 B per token) + k, v (2 048 B each) against one buffer, bytes = 2 x payload; one launch for
+                      the three tensors (what the server tick issues), and as three launches (the reference's call shape);
+      memcpy_cp       replicating pack of k to up to 2 destinations per shard (every shard to the first, every other
+                      shard to the second too) and the unpack into replica planes, bytes = 2 x bytes of live replicas;
+      grad_sum        a third of the rows are main shards with 2 duplicate copies each, bytes = (2 + copies) x rows x
+                      token bytes per main shard."""
     from distca_amd import _lib
-    from distca_amd.ops import a2a_memcpy_non_cp
+    from distca_amd.ops import a2a_memcpy_cp, a2a_memcpy_non_cp, a2a_memcpy_non_cp_multi, pre_a2a_grad_acc
     from distca_amd.workloads import config4_pack
     lay = config4_pack()
     T = lay.num_tokens
+    names = list(lay.token_bytes)
     tens = {n: torch.randint(-32768, 32767, (T, tb // 2), dtype=torch.int16, device=dev).view(torch.bfloat16)
             for n, tb in lay.token_bytes.items()}
     buf = torch.empty(lay.buffer_bytes, dtype=torch.uint8, device=dev)
@@ -92,22 +118,53 @@ def pack_unpack_bench(torch, dev, iters: int = 10):
     payload = sum(T * tb for tb in lay.token_bytes.values())
     res = {}
     for direction, to_buf in (("pack", True), ("unpack", False)):
-        for _ in range(2):
-            for n in tens:
-                a2a_memcpy_non_cp(tens[n], offs[n], lens, to_buf, buffer=buf)
-        torch.cuda.synchronize()
-        _lib.timing_read(_lib.TIMER_MEMCPY_NON_CP)
-        _lib.timing_enable(True)
-        for _ in range(iters):
-            for n in tens:
-                a2a_memcpy_non_cp(tens[n], offs[n], lens, to_buf, buffer=buf)
-        torch.cuda.synchronize()
-        _lib.timing_enable(False)
-        ms, launches = _lib.timing_read(_lib.TIMER_MEMCPY_NON_CP)
-        gbps = 2 * payload * iters / (ms * 1e-3) / 1e9
-        res[direction] = {"GB/s": round(gbps, 1), "frac_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
-                          "ms_per_pass": round(ms / iters, 4), "launches": launches}
+        ms, n1 = _timed(torch, _lib, _lib.TIMER_MEMCPY_NON_CP, lambda: a2a_memcpy_non_cp_multi(
+            [tens[n] for n in names], [offs[n] for n in names], [lens] * len(names), to_buf, buffer=buf), iters)
+        res[direction] = dict(_rate(2 * payload, ms), launches_per_pass=n1)
+        ms3, n3 = _timed(torch, _lib, _lib.TIMER_MEMCPY_NON_CP, lambda: [
+            a2a_memcpy_non_cp(tens[n], offs[n], lens, to_buf, buffer=buf) for n in names], iters)
+        res[direction]["as_separate_launches"] = dict(_rate(2 * payload, ms3), launches_per_pass=n3)
     res["workload"] = f"{lay.name}: {len(lay.seq_tokens)} shards, payload {payload} B per direction"
+
+    # replicating pack / replica-plane unpack of k
+    S, tb = len(lay.seq_tokens), lay.token_bytes["k"]
+    do_shard = np.ones((S, 2), dtype=np.int8)
+    do_shard[1::2, 1] = 0
+    cp_off = np.zeros((2, S), dtype=np.int64)
+    cur = 0
+    for c in range(2):
+        for sidx in range(S):
+            cp_off[c, sidx] = cur
+            if do_shard[sidx, c]:
+                cur += int(lay.seq_tokens[sidx]) * tb
+    live_bytes = cur
+    cp_buf = torch.empty(live_bytes, dtype=torch.uint8, device=dev)
+    d_do, d_off = torch.from_numpy(do_shard).to(dev), torch.from_numpy(cp_off).to(dev)
+    planes = torch.zeros((2, T, tb // 2), dtype=torch.bfloat16, device=dev)
+    ms, _ = _timed(torch, _lib, _lib.TIMER_MEMCPY_CP, lambda: a2a_memcpy_cp(tens["k"], d_do, d_off, lens, True, buffer=cp_buf), iters)
+    res["memcpy_cp_pack"] = dict(_rate(2 * live_bytes, ms), workload=f"k of {T} tokens x {tb} B, {S} shards, {live_bytes / (T * tb):.2f} replicas per shard")
+    ms, _ = _timed(torch, _lib, _lib.TIMER_MEMCPY_CP, lambda: a2a_memcpy_cp(planes, d_do, d_off, lens, False, buffer=cp_buf), iters)
+    res["memcpy_cp_unpack"] = _rate(2 * live_bytes, ms)
+    del planes, cp_buf
+
+    # duplicate-gradient sum: main shards in the first third of the rows, their two copies in the other two thirds
+    main, total = [], 0
+    for n in lay.seq_tokens.tolist():
+        if total + n > T // 3:
+            break
+        main.append(n)
+        total += n
+    m = len(main)
+    seq_lens = torch.tensor(main * 3, dtype=torch.int64, device=dev)
+    num_copies = torch.tensor([2] * m + [0] * (2 * m), dtype=torch.int32, device=dev)
+    starts = np.concatenate([[0], np.cumsum(main)[:-1]]).astype(np.int64)
+    copy_start = np.zeros((3 * m, 2), dtype=np.int64)
+    copy_start[:m, 0] = total + starts
+    copy_start[:m, 1] = 2 * total + starts
+    dk = (torch.randn((3 * total, tb // 2), device=dev) * 0.1).to(torch.bfloat16)
+    d_cs = torch.from_numpy(copy_start).to(dev)
+    ms, _ = _timed(torch, _lib, _lib.TIMER_GRAD_SUM, lambda: pre_a2a_grad_acc(dk, num_copies, d_cs, seq_lens), iters)
+    res["grad_sum"] = dict(_rate(4 * total * tb, ms), workload=f"bf16 [{3 * total}, {tb // 2}]: {m} main shards ({total} rows) with 2 copies each")
     return res
 
 
@@ -186,8 +243,11 @@ def main():
     if not args.no_pack:
         del dq, dk, dv
         pack = pack_unpack_bench(torch, dev)
-        log(f"  pack   {pack['pack']['GB/s']} GB/s ({100 * pack['pack']['frac_hbm_peak']:.1f}% of HBM peak)")
-        log(f"  unpack {pack['unpack']['GB/s']} GB/s ({100 * pack['unpack']['frac_hbm_peak']:.1f}% of HBM peak)")
+        for key in ("pack", "unpack", "memcpy_cp_pack", "memcpy_cp_unpack", "grad_sum"):
+            log(f"  {key:17s} {pack[key]['GB/s']} GB/s ({100 * pack[key]['frac_hbm_peak']:.1f}% of HBM peak)")
+        for key in ("pack", "unpack"):
+            sep = pack[key]["as_separate_launches"]
+            log(f"  {key:17s} as three launches {sep['GB/s']} GB/s ({100 * sep['frac_hbm_peak']:.1f}%)")
 
     cpu = None
     if args.cpu_seconds > 0:

@@ -27,11 +27,22 @@ class CaParams(Structure):
     ]
 
 
+class PackJob(Structure):
+    """struct distca_pack_job (include/distca_ca.h)."""
+    _fields_ = [
+        ("tensor", c_void_p), ("seq_offset", c_void_p), ("seq_tokens", c_void_p), ("copy_seq_mask", c_void_p),
+        ("num_seq", c_int64), ("token_bytes", c_int64), ("num_tokens", c_int64),
+    ]
+
+
+PACK_MAX_JOBS = 4
+
 # name -> (restype, argtypes); every symbol include/distca_ca.h declares
 SYMBOLS = {
     "distca_last_error": (c_char_p, []),
     "distca_abi_version": (c_int, []),
     "distca_memcpy_non_cp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "distca_memcpy_non_cp_multi": (c_int, [POINTER(PackJob), c_int32, c_void_p, c_int, c_void_p]),
     "distca_memcpy_cp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p]),
     "distca_grad_sum": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "distca_ca_fwd_workspace_bytes": (c_int64, [POINTER(CaParams)]),

@@ -15,12 +15,26 @@
 namespace distca {
 namespace {
 
-// 1024-thread workgroups, each streaming one contiguous slice with 4 vectors per thread in
-// flight and non-temporal accesses, reached 5.7 TB/s on a plain 2 GiB copy; 256-thread
-// workgroups and grid-stride forms stayed between 4.5 and 5.4 TB/s.
+// What a plain 3 GiB device-to-device copy reaches on this part, by shape of the kernel (HBM peak 8 TB/s): 1024-thread
+// workgroups over contiguous slices with 4 vectors per lane in flight 69.7 %, with 8 in flight 73 %; 512- and
+// 256-thread workgroups 65-70 %; plain instead of non-temporal loads or stores 66-67 %; hipMemcpyDtoD 59 %.  Best is a
+// workgroup that issues every load of its slice before its first store and then ends (one loop round per slice):
+// 75-76 %; each further round of the same workgroup costs 2-4 %, and a slice that ends in a round of fewer vectors
+// loses more (16 in flight over a slice of one and a half rounds: 68 %).  So a slice is one round where tokens
+// allow, and the last, partial round of a run inside a shard is issued like a whole one with the lanes past the end
+// switched off.  On the 262 144-token q/k/v workload, one launch for the three tensors: 10 vectors per lane
+// (160 KiB slices) 75.4 / 75.3 % packing / unpacking, 16 (256 KiB) 75.0 / 75.5 %, 8 in three rounds 70.7 / 71.7 %,
+// 20 or 24 in one round 73 %, 32 in one round 65 %.
 constexpr int kPackThreads = 1024;
 constexpr int kPackWaves = kPackThreads / 64;
-constexpr int kUnroll = 4;
+#ifndef DISTCA_PACK_UNROLL
+#define DISTCA_PACK_UNROLL 10
+#endif
+#ifndef DISTCA_PACK_SLICE_ROUNDS
+#define DISTCA_PACK_SLICE_ROUNDS 1
+#endif
+constexpr int kUnroll = DISTCA_PACK_UNROLL;
+constexpr int64_t kRoundBytes = (int64_t)kUnroll * kPackThreads * 16;  // bytes a workgroup moves per loop round
 
 // Inclusive block scan of one int64 per thread.
 __device__ __forceinline__ int64_t block_inclusive_scan(int64_t v, int64_t *lds_wave_sums) {
@@ -88,10 +102,18 @@ __device__ __forceinline__ void copy_bytes(uint8_t *__restrict__ dst, const uint
       else d[i + u * kPackThreads] = r[u];
     }
   }
-  for (; i < nvec; i += kPackThreads) {
-    u32x4 r = __builtin_nontemporal_load(s + i);
-    if (STORE_NT) __builtin_nontemporal_store(r, d + i);
-    else d[i] = r;
+  if (i < nvec) {
+    // the last, partial round: every load is issued before the first store, as in a whole round
+    u32x4 r[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (i + u * kPackThreads < nvec) r[u] = __builtin_nontemporal_load(s + i + u * kPackThreads);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (i + u * kPackThreads < nvec) {
+        if (STORE_NT) __builtin_nontemporal_store(r[u], d + i + u * kPackThreads);
+        else d[i + u * kPackThreads] = r[u];
+      }
   }
 }
 
@@ -100,17 +122,10 @@ __device__ __forceinline__ void copy_bytes(uint8_t *__restrict__ dst, const uint
 //   cp:    logical token L in [0, num_tokens*max_cp); the shard list is walked max_cp times,
 //          pass c covering replica c.  Packing reads row L % num_tokens, unpacking writes row L.
 template <bool TO_BUF, bool CP>
-__global__ __launch_bounds__(kPackThreads) void pack_kernel(
-    uint8_t *__restrict__ tensor, uint8_t *__restrict__ buffer, const int64_t *__restrict__ seq_offset,
-    const int64_t *__restrict__ seq_tokens, const int8_t *__restrict__ mask, int64_t num_seq, int64_t token_bytes,
-    int64_t num_tokens, int32_t max_cp, int64_t tokens_per_wg) {
-  __shared__ int64_t lds_scratch[kPackWaves + 2];
-  const int64_t logical_tokens = CP ? num_tokens * max_cp : num_tokens;
-  int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg;
-  int64_t t1 = t0 + tokens_per_wg;
-  if (t1 > logical_tokens) t1 = logical_tokens;
-  if (t0 >= t1) return;
-
+__device__ __forceinline__ void pack_slice(uint8_t *__restrict__ tensor, uint8_t *__restrict__ buffer,
+                                           const int64_t *__restrict__ seq_offset, const int64_t *__restrict__ seq_tokens,
+                                           const int8_t *__restrict__ mask, int64_t num_seq, int64_t token_bytes,
+                                           int64_t num_tokens, int32_t max_cp, int64_t t0, int64_t t1, int64_t *lds_scratch) {
   int64_t cp = 0, pos = t0, total = 0;
   if (CP) {
     Cursor c = locate(seq_tokens, num_seq, 0, true, lds_scratch);
@@ -162,6 +177,55 @@ __global__ __launch_bounds__(kPackThreads) void pack_kernel(
       if (++cp >= max_cp) break;
     }
   }
+}
+
+// One kernel for the plain and the replicating ("cp") form.
+//   plain: logical token L in [0, num_tokens) is row L of the tensor; shard list walked once.
+//   cp:    logical token L in [0, num_tokens*max_cp); the shard list is walked max_cp times,
+//          pass c covering replica c.  Packing reads row L % num_tokens, unpacking writes row L.
+template <bool TO_BUF, bool CP>
+__global__ __launch_bounds__(kPackThreads) void pack_kernel(
+    uint8_t *__restrict__ tensor, uint8_t *__restrict__ buffer, const int64_t *__restrict__ seq_offset,
+    const int64_t *__restrict__ seq_tokens, const int8_t *__restrict__ mask, int64_t num_seq, int64_t token_bytes,
+    int64_t num_tokens, int32_t max_cp, int64_t tokens_per_wg) {
+  __shared__ int64_t lds_scratch[kPackWaves + 2];
+  const int64_t logical_tokens = CP ? num_tokens * max_cp : num_tokens;
+  int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg;
+  int64_t t1 = t0 + tokens_per_wg;
+  if (t1 > logical_tokens) t1 = logical_tokens;
+  if (t0 >= t1) return;
+  pack_slice<TO_BUF, CP>(tensor, buffer, seq_offset, seq_tokens, mask, num_seq, token_bytes, num_tokens, max_cp, t0, t1, lds_scratch);
+}
+
+// Several tensors against one buffer in one launch (the q, k and v of a tick): workgroups [first_wg, first_wg of the
+// next job) serve job j.  One launch has one tail instead of three, and the small tensors' slices fill the gaps
+// the large one leaves.
+constexpr int kMaxPackJobs = DISTCA_PACK_MAX_JOBS;
+struct PackJob {
+  uint8_t *tensor;
+  const int64_t *seq_offset, *seq_tokens;
+  const int8_t *mask;
+  int64_t num_seq, token_bytes, num_tokens, tokens_per_wg;
+  int32_t first_wg;
+};
+struct PackJobs {
+  PackJob job[kMaxPackJobs];
+  int32_t n;
+};
+template <bool TO_BUF>
+__global__ __launch_bounds__(kPackThreads) void pack_multi_kernel(PackJobs jobs, uint8_t *__restrict__ buffer) {
+  __shared__ int64_t lds_scratch[kPackWaves + 2];
+  int j = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxPackJobs; ++i)
+    if (i < jobs.n && (int)blockIdx.x >= jobs.job[i].first_wg) j = i;
+  const PackJob &jb = jobs.job[j];
+  int64_t t0 = (int64_t)((int)blockIdx.x - jb.first_wg) * jb.tokens_per_wg;
+  int64_t t1 = t0 + jb.tokens_per_wg;
+  if (t1 > jb.num_tokens) t1 = jb.num_tokens;
+  if (t0 >= t1) return;
+  pack_slice<TO_BUF, false>(jb.tensor, buffer, jb.seq_offset, jb.seq_tokens, TO_BUF ? jb.mask : nullptr, jb.num_seq, jb.token_bytes,
+                            jb.num_tokens, 1, t0, t1, lds_scratch);
 }
 
 template <typename T>
@@ -253,15 +317,17 @@ __global__ __launch_bounds__(kPackThreads) void grad_sum_kernel(T *__restrict__ 
   }
 }
 
+// Tokens per workgroup slice: kSliceRounds loop rounds (one: 160 KiB at 10 vectors per lane), rounded to whole
+// tokens; never below one round.
+constexpr int kSliceRounds = DISTCA_PACK_SLICE_ROUNDS;
 int64_t slice_tokens(int64_t logical_tokens, int64_t token_bytes, int *grid) {
-  // 16 slices per CU (4096 on MI355X: a power-of-two count spreads the slices evenly over
-  // the memory channels; measured best among 1..16 per CU); never cut slices below 256 KiB.
-  int64_t g = (int64_t)num_compute_units() * 16;
-  int64_t min_tok = (262144 + token_bytes - 1) / token_bytes;
-  int64_t per = (logical_tokens + g - 1) / g;
-  if (per < min_tok) per = min_tok;
+  int64_t bytes = kSliceRounds * kRoundBytes;
+  const int64_t total = logical_tokens * token_bytes, want = (int64_t)num_compute_units() * 4;
+  while (bytes > kRoundBytes && total / bytes < want) bytes -= kRoundBytes;
+  int64_t per = (bytes + token_bytes / 2) / token_bytes;
   if (per < 1) per = 1;
-  *grid = (int)((logical_tokens + per - 1) / per);
+  const int64_t g = (logical_tokens + per - 1) / per;
+  *grid = (int)(g < 0x7fffffff ? g : 0x7fffffff);
   return per;
 }
 
@@ -291,6 +357,43 @@ extern "C" int distca_memcpy_non_cp(void *tensor, void *buffer, const int64_t *s
     hipLaunchKernelGGL((pack_kernel<false, false>), dim3(grid), dim3(kPackThreads), 0, s, t, b, seq_offset, seq_tokens,
                        (const int8_t *)nullptr, num_seq, token_bytes, num_tokens, 1, per);
   return check_launch("memcpy_non_cp");
+}
+
+extern "C" int distca_memcpy_non_cp_multi(const distca_pack_job *jobs, int32_t num_jobs, void *buffer, int to_buffer, void *stream) {
+  if (num_jobs < 0 || num_jobs > kMaxPackJobs) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: %d jobs (0..%d)", num_jobs, kMaxPackJobs);
+  if (num_jobs == 0) return DISTCA_OK;
+  if (!jobs) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: null job list");
+  PackJobs pj;
+  pj.n = 0;
+  int64_t wg = 0;
+  for (int i = 0; i < num_jobs; ++i) {
+    const distca_pack_job &in = jobs[i];
+    if (in.num_seq < 0 || in.num_tokens < 0 || in.token_bytes < 0) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: job %d: negative size", i);
+    if (in.num_tokens == 0 || in.num_seq == 0 || in.token_bytes == 0) continue;
+    if (!in.tensor || !buffer || !in.seq_offset || !in.seq_tokens) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: job %d: null pointer", i);
+    if (in.token_bytes % 16) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: job %d: token_bytes=%lld is not a multiple of 16", i, (long long)in.token_bytes);
+    if (!aligned16(in.tensor) || !aligned16(buffer)) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: job %d: tensor/buffer must be 16-byte aligned", i);
+    if (in.num_tokens >= (1ll << 31)) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: job %d: num_tokens must be < 2^31", i);
+    PackJob &o = pj.job[pj.n++];
+    int grid;
+    o.tokens_per_wg = slice_tokens(in.num_tokens, in.token_bytes, &grid);
+    o.tensor = (uint8_t *)in.tensor;
+    o.seq_offset = in.seq_offset;
+    o.seq_tokens = in.seq_tokens;
+    o.mask = in.copy_seq_mask;
+    o.num_seq = in.num_seq;
+    o.token_bytes = in.token_bytes;
+    o.num_tokens = in.num_tokens;
+    o.first_wg = (int32_t)wg;
+    wg += grid;
+    if (wg > 0x7fffffff) return fail(DISTCA_E_INVALID, "memcpy_non_cp_multi: grid too large");
+  }
+  if (pj.n == 0) return DISTCA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  ScopedTimer timer(DISTCA_TIMER_MEMCPY_NON_CP, s);
+  if (to_buffer) hipLaunchKernelGGL((pack_multi_kernel<true>), dim3((unsigned)wg), dim3(kPackThreads), 0, s, pj, (uint8_t *)buffer);
+  else hipLaunchKernelGGL((pack_multi_kernel<false>), dim3((unsigned)wg), dim3(kPackThreads), 0, s, pj, (uint8_t *)buffer);
+  return check_launch("memcpy_non_cp_multi");
 }
 
 extern "C" int distca_memcpy_cp(void *tensor, void *buffer, const int8_t *do_shard, const int64_t *seq_offset,

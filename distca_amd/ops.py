@@ -74,6 +74,44 @@ def a2a_memcpy_non_cp(
     return None
 
 
+def a2a_memcpy_non_cp_multi(tensors, nvshmem_offsets, shard_tokens, to_nvshmem: bool, shard_do_copy_masks=None, *,
+                            buffer: torch.Tensor):
+    """Several a2a_memcpy_non_cp calls against one buffer as a single launch: tensors[i] with nvshmem_offsets[i],
+    shard_tokens[i] and (packing only) shard_do_copy_masks[i].  What the reference does with consecutive calls for
+    the q, k and v of a tick (distca/runtime/attn_kernels/dispatch.py:39-56,60-94); the result is the same bytes."""
+    n = len(tensors)
+    if not (len(nvshmem_offsets) == len(shard_tokens) == n) or (shard_do_copy_masks is not None and len(shard_do_copy_masks) != n):
+        raise RuntimeError("a2a_memcpy_non_cp_multi: one offset tensor, one length tensor and at most one mask per tensor")
+    if n > _lib.PACK_MAX_JOBS:
+        raise RuntimeError(f"a2a_memcpy_non_cp_multi: at most {_lib.PACK_MAX_JOBS} tensors per launch")
+    if n == 0:
+        return None
+    if not buffer.is_cuda:
+        raise RuntimeError("tensor buffer must be on CUDA")
+    jobs = (_lib.PackJob * n)()
+    for i in range(n):
+        t, off, tok = tensors[i], nvshmem_offsets[i], shard_tokens[i]
+        _check_tensor(2, t, "tensor")
+        _check_tensor(1, off, "seq_nvshmem_offset")
+        _check_tensor(1, tok, "seq_tokens")
+        _check_dtype(off, torch.int64, "seq_nvshmem_offset")
+        _check_dtype(tok, torch.int64, "seq_tokens")
+        if tok.size(0) != off.size(0):
+            raise RuntimeError("seq_tokens must be of shape (num_sequence,)")
+        mask = shard_do_copy_masks[i] if shard_do_copy_masks is not None else None
+        if mask is not None:
+            _check_tensor(1, mask, "copy_seq_mask")
+            _check_dtype(mask, torch.int8, "copy_seq_mask")
+            if mask.size(0) != off.size(0):
+                raise RuntimeError("copy_seq_mask must be of shape (num_sequence,)")
+        jobs[i] = _lib.PackJob(t.data_ptr(), off.data_ptr(), tok.data_ptr(), mask.data_ptr() if mask is not None else None,
+                               off.size(0), t.size(1) * t.element_size(), t.size(0))
+    with torch.cuda.device(buffer.device):
+        rc = _lib.load().distca_memcpy_non_cp_multi(jobs, n, buffer.data_ptr(), 1 if to_nvshmem else 0, _stream())
+    _lib.check(rc, "a2a_memcpy_non_cp_multi")
+    return None
+
+
 def a2a_memcpy_cp(
     tensor: torch.Tensor, do_shard: torch.Tensor,
     nvshmem_offset: torch.Tensor, shard_tokens: torch.Tensor,

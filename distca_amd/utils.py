@@ -1,27 +1,30 @@
-"""Small host helpers shared by the op wrappers (same names and meaning as
-distca/runtime/utils.py:8-35 in the reference)."""
+"""Host helpers shared by the op wrappers.  The three public names and their meaning are those of
+distca/runtime/utils.py:8-35 in the reference, so that code written against it keeps working."""
 from __future__ import annotations
 
 import torch
 
-_INT4_BYTES = 16
+TRANSPORT_ALIGN = 16  # bytes: one 128-bit vector, the unit the pack kernels move
+
+
+def round_up(n: int, unit: int = TRANSPORT_ALIGN) -> int:
+    return -(-int(n) // unit) * unit
 
 
 def size_pad_by_int4(hidden_size: int, itemsize: int):
-    """(padded element count, pad element count) so that a row is a multiple of 16 bytes."""
-    hidden_bytes = hidden_size * itemsize
-    if hidden_bytes % _INT4_BYTES != 0:
-        hidden_bytes += _INT4_BYTES - (hidden_bytes % _INT4_BYTES)
-    hidden_size_pad = hidden_bytes // itemsize
-    return hidden_size_pad, hidden_size_pad - hidden_size
+    """A token row of `hidden_size` elements of `itemsize` bytes, padded so that the row is a whole number of
+    128-bit vectors: returns (padded element count, elements of padding)."""
+    padded = round_up(hidden_size * itemsize) // itemsize
+    return padded, padded - hidden_size
 
 
-def prepend_zero_fn(tensor: torch.Tensor, dim: int = 0):
-    zero = torch.zeros_like(tensor.select(dim, 0)).unsqueeze(dim)
-    return torch.cat([zero, tensor], dim=dim)
+def prepend_zero_fn(tensor: torch.Tensor, dim: int = 0) -> torch.Tensor:
+    """`tensor` with one zero slice put in front along `dim` (a cumulative sum turned into cu_seqlens)."""
+    shape = list(tensor.shape)
+    shape[dim] = 1
+    return torch.cat((tensor.new_zeros(shape), tensor), dim=dim)
 
 
 def exclusive_cumsum(tensor: torch.Tensor, dim: int = 0) -> torch.Tensor:
-    cumsum = tensor.cumsum(dim=dim)
-    zero = torch.zeros_like(tensor.select(dim, 0))
-    return torch.cat([zero.unsqueeze(dim), cumsum.narrow(dim, 0, cumsum.size(dim) - 1)], dim=dim)
+    """Sum of the elements before each position along `dim`: the inclusive sum less the element itself."""
+    return tensor.cumsum(dim=dim) - tensor

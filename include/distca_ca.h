@@ -66,6 +66,26 @@ int distca_memcpy_non_cp(void *tensor, void *buffer,
                          int64_t token_bytes, int64_t num_tokens, int to_buffer,
                          void *stream);
 
+/* Several tensors packed into / unpacked from one buffer by one launch: what the
+ * reference does with consecutive launch_memcpy_non_cp calls for the q, k and v of a
+ * tick (post_a2a_qkv, distca/runtime/attn_kernels/dispatch.py:60-94; pre_a2a_qkv in
+ * backward, :39-56).  Each job has the meaning of one distca_memcpy_non_cp call with
+ * the same fields; results are identical to making those calls one after another, the
+ * jobs' byte ranges in the buffer being disjoint.  At most DISTCA_PACK_MAX_JOBS jobs;
+ * jobs with no tokens are skipped. */
+#define DISTCA_PACK_MAX_JOBS 4
+typedef struct distca_pack_job {
+  void *tensor;
+  const int64_t *seq_offset;   /* device, int64 [num_seq] */
+  const int64_t *seq_tokens;   /* device, int64 [num_seq] */
+  const int8_t *copy_seq_mask; /* device, int8 [num_seq] or NULL; packing only */
+  int64_t num_seq;
+  int64_t token_bytes;
+  int64_t num_tokens;
+} distca_pack_job;
+int distca_memcpy_non_cp_multi(const distca_pack_job *jobs, int32_t num_jobs,
+                               void *buffer, int to_buffer, void *stream);
+
 /* Replaces launch_memcpy_cp (csrc/core/memcpy.cu:285-343; kernel :77-155) as
  * reached through fast_a2a_memcpy_cp[_debug] (all_to_all.cpp:116-179,243-254).
  * Logical shard (c, s), c < max_cp, s < num_seq, is live iff

@@ -50,6 +50,57 @@ def test_non_cp_pack_unpack(cuda, hidden, dtype, nshard):
     assert np.array_equal(dst.view(torch.uint8).reshape(T, tb).cpu().numpy(), exp_t)
 
 
+@pytest.mark.parametrize("scale", [1, 60])
+def test_several_tensors_in_one_launch(cuda, scale):
+    """a2a_memcpy_non_cp_multi (q, k, v of a tick against one buffer in one launch) leaves the bytes the oracle leaves
+    after three separate copies: packing with and without per-shard masks, then unpacking into poisoned tensors.
+    `scale` 60 makes shards of up to 2 400 tokens (19 MB): slices of several loop rounds that cross shard ends."""
+    from distca_amd.ops import a2a_memcpy_non_cp_multi
+    rng = np.random.default_rng(500 + scale)
+    hiddens = [4096, 1024, 1024, 520]                      # bf16 q, k, v and an odd fourth tensor (1040-byte tokens)
+    shard_counts = [11, 17, 17, 3]
+    lens = [(rng.integers(0, 40, size=n) * scale).astype(np.int64) for n in shard_counts]
+    for l in lens:
+        l[rng.integers(0, len(l))] += 5
+    lens[2] = lens[1].copy()
+    tbs = [h * 2 for h in hiddens]
+    offs, base = [], 0
+    for l, tb in zip(lens, tbs):
+        o, n = _layout(rng, l, tb)
+        offs.append(o + base)
+        base += n
+    srcs = [rng.integers(0, 256, size=(int(l.sum()), tb), dtype=np.uint8) for l, tb in zip(lens, tbs)]
+    masks = [(rng.random(len(l)) < 0.6).astype(np.int8) for l in lens]
+    dev = lambda a: torch.from_numpy(a).to(cuda)
+    d_srcs = [dev(a).view(torch.bfloat16) for a in srcs]
+    d_offs, d_lens, d_masks = [dev(o) for o in offs], [dev(l) for l in lens], [dev(m) for m in masks]
+    for use_mask in (True, False):
+        buf0 = rng.integers(0, 256, size=base, dtype=np.uint8)
+        exp = buf0.copy()
+        for a, o, l, m, tb in zip(srcs, offs, lens, masks, tbs):
+            fa2a.copy_non_cp(a, exp, o, l, m if use_mask else None, True)
+        dbuf = dev(buf0.copy())
+        print(f"multi pack scale={scale} mask={use_mask} buffer {base} B", flush=True)
+        a2a_memcpy_non_cp_multi(d_srcs, d_offs, d_lens, True, d_masks if use_mask else None, buffer=dbuf)
+        torch.cuda.synchronize()
+        assert np.array_equal(dbuf.cpu().numpy(), exp)
+    dsts = [torch.full(a.shape, 0x5A, dtype=torch.uint8, device=cuda).view(torch.bfloat16) for a in srcs]
+    print(f"multi unpack scale={scale}", flush=True)
+    a2a_memcpy_non_cp_multi(dsts, d_offs, d_lens, False, d_masks, buffer=dbuf)     # masks are ignored when unpacking
+    torch.cuda.synchronize()
+    for a, d in zip(srcs, dsts):
+        assert np.array_equal(d.view(torch.uint8).cpu().numpy(), a)
+    # fewer jobs, one of them empty
+    empty = torch.empty((0, 1024), dtype=torch.bfloat16, device=cuda)
+    z = torch.zeros(0, dtype=torch.int64, device=cuda)
+    dbuf2 = dev(np.zeros(base, dtype=np.uint8))
+    a2a_memcpy_non_cp_multi([d_srcs[0], empty], [d_offs[0], z], [d_lens[0], z], True, buffer=dbuf2)
+    torch.cuda.synchronize()
+    exp2 = np.zeros(base, dtype=np.uint8)
+    fa2a.copy_non_cp(srcs[0], exp2, offs[0], lens[0], None, True)
+    assert np.array_equal(dbuf2.cpu().numpy(), exp2)
+
+
 @pytest.mark.parametrize("max_cp", [1, 3])
 def test_cp_pack_unpack(cuda, max_cp):
     from distca_amd.ops import a2a_memcpy_cp
