@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libdistca_ca.so")
-SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip"]
+SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-x", "hip",
@@ -36,8 +36,20 @@ def _hipcc() -> str:
     return exe
 
 
+# Flags a source must not be compiled with.  attn_bwd_dkdv64.hip wants the compiler's default MFMA form (results in
+# the accumulation registers) for its 256 dK/dV accumulators; the accumulators its vector ALU touches are pinned
+# to vector registers in the source.
+DROP_FLAGS = {"attn_bwd_dkdv64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def _compile(src: str, obj: str, extra: list[str]) -> None:
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    flags = list(HIPCC_FLAGS)
+    drop = DROP_FLAGS.get(src, [])
+    for i in range(len(flags) - len(drop) + 1):
+        if drop and flags[i:i + len(drop)] == drop:
+            del flags[i:i + len(drop)]
+            break
+    cmd = [_hipcc(), *flags, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the gfx950 feature name and says so; drop that line
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

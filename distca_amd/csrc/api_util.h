@@ -45,6 +45,6 @@ int num_compute_units();
 // may both do the set-up, which is idempotent).
 bool device_setup_pending(int slot);
 void device_setup_done(int slot);
-enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotCount = 2 };
+enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotBwdLds64 = 2, kSlotCount = 3 };
 
 }  // namespace distca

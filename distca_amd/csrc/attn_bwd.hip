@@ -37,6 +37,7 @@
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 #include "api_util.h"
+#include "attn_bwd.h"
 #include "attn_cfg.h"
 #include "common.h"
 
@@ -45,6 +46,9 @@
 namespace distca {
 namespace {
 
+#ifndef DISTCA_DKDV64
+#define DISTCA_DKDV64 1
+#endif
 constexpr int kPitch = 272;  // bytes per 128-element bf16 row in LDS
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -69,27 +73,6 @@ constexpr int kStatBytes = 3 * kBM * 4;           // per stage: lse2, dscaled, l
 constexpr int kBwdLds = kKsOff + kBN * kPitch;
 static_assert(kStatOff + kStages * kStatBytes <= kBwdLds, "tile ring must fit in the K staging region");
 static_assert(kBwdLds <= 160 * 1024, "LDS budget");
-
-struct BwdArgs {
-  const __bf16 *q, *k, *v, *dout;
-  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and -delta
-  __bf16 *dq, *dk, *dv;
-  float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
-  const int32_t *cu_q, *cu_k, *kv_off;
-  const int32_t *sched;
-  int32_t *tickets;  // one counter per kv head (sched.h)
-  const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
-  int32_t sched_items_off;
-  int32_t hq, hkv, group, total_q;
-  uint32_t group_magic;  // ceil(2^32 / group), 0 when group == 1: n / group == umulhi(n, magic) for n * group < 2^32
-  int32_t causal;
-  float scale;
-  // Where the query-side tokens live: q and dout point at the first byte of their part of token 0 of a
-  // region in which token t of task b starts at off[b] + t * tok_bytes (off == nullptr: the packed
-  // tensors, off[b] = cu_q[b] * tok_bytes); head h at + h * 256 bytes.  dq likewise.
-  const int64_t *qs_task_off, *dq_task_off;
-  int64_t qs_tok_bytes, dq_tok_bytes;
-};
 
 template <bool ALIAS>
 __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) {
@@ -1004,10 +987,15 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
+#if DISTCA_DKDV64
+    rc = launch_dkdv64(a, grid, use_acc, s);
+    if (rc) return rc;
+#else
     if (use_acc)
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
     else
       hipLaunchKernelGGL((ca_bwd_dkdv_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
+#endif
   }
   // ---- dQ: one workgroup per (task, block of query rows, kv head)
   {
