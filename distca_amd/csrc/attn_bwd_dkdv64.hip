@@ -45,8 +45,8 @@ constexpr int kVPitch = 272;             // resident V rows (padded: 128-bit row
 constexpr int kVOff = kStatOff + kStages * kStatBytes;
 constexpr int kLds = kVOff + kBN * kVPitch;
 static_assert(kLds <= 160 * 1024, "LDS budget");
-#ifndef DISTCA_ABL
-#define DISTCA_ABL 0
+#ifndef DISTCA_RAWBAR
+#define DISTCA_RAWBAR 1
 #endif
 constexpr int kLoadsPerBlock = 6;        // vector-memory instructions a wave issues per block
 constexpr float kLog2e = 1.4426950408889634f;
@@ -393,16 +393,18 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   auto advance = [&](int p) {
     // block p has landed when at most the loads of block p + 1 are still on their way (requests are made for blocks
     // past the end as well, from the zero row, which keeps that count fixed)
-#if DISTCA_ABL != 1
     wait_vm<kLoadsPerBlock>();
-#endif
-#if DISTCA_ABL != 2
+#if DISTCA_RAWBAR
+    // the bare barrier instruction: what it orders are the LDS-direct loads, which the counted wait above covers;
+    // __syncthreads() would also wait for this wave's own LDS reads in flight
+    fence();
+    asm volatile("s_barrier" ::: "memory");
+    fence();
+#else
     __syncthreads();
 #endif
     // stage (p + 2) % 4 was last read for block p - 2, which every wave left before this barrier
-#if DISTCA_ABL != 1
     issue_tile((p + 2) % kStages, top - 1 - (p + 2));
-#endif
   };
   int p = 0;
   for (; p < niter; ++p) {
