@@ -18,7 +18,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .ops import a2a_memcpy_non_cp, pre_a2a_grad_acc
+from .ops import a2a_memcpy_non_cp, a2a_memcpy_non_cp_multi, pre_a2a_grad_acc
 from .utils import size_pad_by_int4
 from .dispatch import (post_a2a_attn_out, post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_grad_resend_qkv,
                        pre_a2a_attn_out_with_lse, pre_a2a_qkv)
@@ -244,6 +244,28 @@ def core_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen
 # between "receive buffer holds this tick's shards" and "send buffer holds the reply".
 # ---------------------------------------------------------------------------------------
 @dataclass
+class SharedKVOnDevice:
+    """metadata.SharedKVLayout as the server tick uses it: per stored shard its tokens and the byte offsets it is
+    unpacked from (and, in backward, its gradient is packed to); per task the first store row of its prefix."""
+    store_tokens: Tensor          # int64 [stored shards]
+    k_offset: Tensor              # int64 [stored shards] into the receive buffer
+    v_offset: Tensor
+    kv_task_offsets: Tensor       # int32 [tasks]
+    num_rows: int
+    k_grad_offset: Optional[Tensor] = None   # int64 [stored shards] into the send buffer (backward)
+    v_grad_offset: Optional[Tensor] = None
+
+    @classmethod
+    def build(cls, layout, k_entry_offset: Tensor, v_entry_offset: Tensor, device, k_grad_entry_offset: Tensor = None,
+              v_grad_entry_offset: Tensor = None) -> "SharedKVOnDevice":
+        """`*_entry_offset`: host int64 tensors with one byte offset per K/V entry (aliases of a shard hold the same)."""
+        pick = lambda t: None if t is None else t.cpu()[layout.entry_of_stored].to(device=device, dtype=torch.int64)
+        return cls(layout.store_tokens.to(device), pick(k_entry_offset), pick(v_entry_offset),
+                   layout.kv_task_offsets.to(device=device, dtype=torch.int32), layout.num_rows,
+                   pick(k_grad_entry_offset), pick(v_grad_entry_offset))
+
+
+@dataclass
 class ServerFwdMeta:
     """Receive-side layout of q/k/v shards and send-side layout of the reply."""
     q_recv_seq_tokens: Tensor      # int64 [nq_shards]
@@ -255,6 +277,7 @@ class ServerFwdMeta:
     out_send_offset: Tensor        # int64 byte offsets into the send buffer ([out | lse] tokens)
     recv_q_shape: Tuple[int, int]  # (Tq, Hq*D)
     recv_k_shape: Tuple[int, int]  # (Tk, Hkv*D)
+    shared_kv: Optional[SharedKVOnDevice] = None   # when given, the in-place tick keeps one copy of every K/V shard
 
 
 def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdMeta, fa_params: PackedSeqParams,
@@ -268,17 +291,25 @@ def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdM
     softmax_lse [Hq,T]) are returned for the caller's own use.  Both leave the same bytes in the
     send buffer."""
     dev = recv_buffer.device
-    recv_k = torch.empty(meta.recv_k_shape, dtype=dtype, device=dev)
-    recv_v = torch.empty_like(recv_k)
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
+    shared = meta.shared_kv if in_place and dtype == torch.bfloat16 else None
+    k_rows = shared.num_rows if shared is not None else meta.recv_k_shape[0]
+    recv_k = torch.empty((k_rows, meta.recv_k_shape[1]), dtype=dtype, device=dev)
+    recv_v = torch.empty_like(recv_k)
     if in_place and dtype == torch.bfloat16:
-        a2a_memcpy_non_cp(recv_k, meta.k_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
-        a2a_memcpy_non_cp(recv_v, meta.v_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
-        tq, tk = int(meta.recv_q_shape[0]), int(meta.recv_k_shape[0])
+        kv_off = getattr(fa_params, "kv_task_offsets", None)
+        if shared is not None:
+            # one copy of every K/V shard, documents contiguous: every task reads its prefix in place
+            a2a_memcpy_non_cp_multi([recv_k, recv_v], [shared.k_offset, shared.v_offset], [shared.store_tokens] * 2, False,
+                                    buffer=recv_buffer)
+            kv_off = shared.kv_task_offsets
+        else:
+            a2a_memcpy_non_cp_multi([recv_k, recv_v], [meta.k_recv_offset, meta.v_recv_offset], [meta.k_recv_seq_tokens] * 2,
+                                    False, buffer=recv_buffer)
+        tq, tk = int(meta.recv_q_shape[0]), int(k_rows)
         scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
         lib = _lib.load()
         cu_q, cu_k = fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv
-        kv_off = getattr(fa_params, "kv_task_offsets", None)
         assert fa_args.causal and fa_args.window_size == (-1, -1) and fa_args.dropout_p == 0.0
         p = _params(cu_q.shape[0] - 1, tq, tk, hq, hkv, d, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, scale,
                     fa_args.causal, False)
@@ -326,6 +357,7 @@ class ServerBwdMeta:
     attn_out_shape: Tuple[int, int]
     lse_shape: Tuple[int, int]     # (T, Hq)
     k_shape: Tuple[int, int]
+    shared_kv: Optional[SharedKVOnDevice] = None
 
 
 def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwdMeta, fa_args: FlashAttnArgs,
@@ -340,13 +372,21 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
     before.  Returns (None, dk, dv) then, else (dq, dk, dv).  Both leave the same bytes in the send
     buffer."""
     dev = recv_buffer.device
-    recv_k = torch.empty(meta.k_shape, dtype=dtype, device=dev)
-    recv_v = torch.empty_like(recv_k)
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
-    if in_place and (hq * 4) % 16 == 0 and dtype == torch.bfloat16:
-        a2a_memcpy_non_cp(recv_k, meta.k_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
-        a2a_memcpy_non_cp(recv_v, meta.v_recv_offset, meta.k_recv_seq_tokens, False, buffer=recv_buffer)
-        tq, tk = int(meta.attn_out_shape[0]), int(meta.k_shape[0])
+    in_place = in_place and (hq * 4) % 16 == 0 and dtype == torch.bfloat16
+    # summed dK/dV of shared rows come from float atomics: not when the caller insists on a deterministic backward
+    shared = meta.shared_kv if in_place and not fa_args.deterministic else None
+    k_rows = shared.num_rows if shared is not None else meta.k_shape[0]
+    recv_k = torch.empty((k_rows, meta.k_shape[1]), dtype=dtype, device=dev)
+    recv_v = torch.empty_like(recv_k)
+    if in_place:
+        if shared is not None:
+            a2a_memcpy_non_cp_multi([recv_k, recv_v], [shared.k_offset, shared.v_offset], [shared.store_tokens] * 2, False,
+                                    buffer=recv_buffer)
+        else:
+            a2a_memcpy_non_cp_multi([recv_k, recv_v], [meta.k_recv_offset, meta.v_recv_offset], [meta.k_recv_seq_tokens] * 2,
+                                    False, buffer=recv_buffer)
+        tq, tk = int(meta.attn_out_shape[0]), int(k_rows)
         scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
         lib = _lib.load()
         p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_kv, scale, fa_args.causal,
@@ -365,12 +405,19 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
         with torch.cuda.device(dev):
             rc = lib.distca_ca_bwd_tokens(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), req_tok, recv_k.data_ptr(),
                                           recv_v.data_ptr(), send_buffer.data_ptr(), meta.q_grad_send_offset.data_ptr(), row,
-                                          dk.data_ptr(), dv.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_kv.data_ptr(), None,
+                                          dk.data_ptr(), dv.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_kv.data_ptr(),
+                                          shared.kv_task_offsets.data_ptr() if shared is not None else None,
                                           ctypes.byref(p), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
         _lib.check(rc, "ca_server_backward")
-        for g, off in ((dk, meta.k_grad_send_offset), (dv, meta.v_grad_send_offset)):
+        if shared is not None:
+            # every stored shard holds the gradient summed over the tasks that read it: one pack, no duplicates to add up
+            a2a_memcpy_non_cp_multi([dk, dv], [shared.k_grad_offset, shared.v_grad_offset], [shared.store_tokens] * 2, True,
+                                    buffer=send_buffer)
+            return None, dk, dv
+        for g in (dk, dv):
             pre_a2a_grad_acc(g, meta.num_copies, meta.copy_start_id, meta.k_grad_send_seq_tokens)
-            a2a_memcpy_non_cp(g, off, meta.k_grad_send_seq_tokens, True, shard_do_copy_mask=meta.main_copy_mask, buffer=send_buffer)
+        a2a_memcpy_non_cp_multi([dk, dv], [meta.k_grad_send_offset, meta.v_grad_send_offset], [meta.k_grad_send_seq_tokens] * 2,
+                                True, [meta.main_copy_mask] * 2, buffer=send_buffer)
         return None, dk, dv
     (dout, out, lse, q, recv_k, recv_v) = post_a2a_attn_out_grad_resend_qkv(
         meta.attn_out_shape, meta.lse_shape, meta.attn_out_shape, torch.float32, recv_k, recv_v, None,
@@ -400,7 +447,8 @@ def fused_comm_attn_forward(recv_buffer: Tensor, send_buffer: Tensor, packed_seq
     q_off, k_off, v_off = qkv.recv_memcpy_metadata
     meta = ServerFwdMeta(qkv.seq_lens[0].recv_seqlens, qkv.seq_lens[1].recv_seqlens, q_off, k_off, v_off,
                          out.seq_lens[0].send_seqlens, out.send_memcpy_metadata[0],
-                         tuple(qkv.tensor_shape[0].recv_shape), tuple(qkv.tensor_shape[1].recv_shape))
+                         tuple(qkv.tensor_shape[0].recv_shape), tuple(qkv.tensor_shape[1].recv_shape),
+                         shared_kv=getattr(packed_seq_params, "shared_kv_fwd", None))
     return ca_server_forward(recv_buffer, send_buffer, meta, packed_seq_params, fa_args, dtype)
 
 
@@ -418,7 +466,7 @@ def fused_comm_attn_backward(recv_buffer: Tensor, send_buffer: Tensor, packed_se
     meta = ServerBwdMeta(req.seq_lens[0].recv_seqlens, req.seq_lens[1].recv_seqlens, q_off, k_off, v_off,
                          grad.seq_lens[0].send_seqlens, grad.seq_lens[1].send_seqlens, gq_off, gk_off, gv_off,
                          d.main_copy_mask, d.num_copies, d.copy_start_id, (tq, hq_d), (tq, fa_args.num_heads_q),
-                         tuple(req.tensor_shape[1].recv_shape))
+                         tuple(req.tensor_shape[1].recv_shape), shared_kv=getattr(packed_seq_params, "shared_kv_bwd", None))
     return ca_server_backward(recv_buffer, send_buffer, meta, fa_args, bwd.cu_seqlens_q, bwd.cu_seqlens_kv,
                               bwd.max_seqlen_q, bwd.max_seqlen_kv, dtype)
 

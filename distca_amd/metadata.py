@@ -151,6 +151,80 @@ def get_attn_metadata(seqlens_q, seqlens_kv=None, get_packed_seq_params: bool = 
 
 
 @dataclass
+class SharedKVLayout:
+    """One stored copy of every K/V shard the tasks of a tick read, the shards of a document side by side
+    in document order, so that every task finds its whole prefix as one run of rows (kv_task_offsets) and
+    nothing is copied once per task.  The reference materialises the prefix of every task
+    (compute_metadata.py:429-448: one recv entry per (task, shard), aliased in the buffer) and sums the
+    gradients of the copies afterwards (inplace_grad_sum_kernel); with this layout the attention kernels
+    read the one copy and leave summed dK/dV in it."""
+    store_tokens: Tensor      # int64 [stored shards]: tokens of each, in store order
+    entry_of_stored: Tensor   # int64 [stored shards]: the K/V entry (first of its aliases) it is unpacked from
+    kv_task_offsets: Tensor   # int32 [tasks]: first store row of each task's prefix
+    num_rows: int
+
+
+def shared_kv_layout(task_kv_lens: Sequence[int], entry_tokens: Sequence[int], entry_key: Sequence[int]) -> Optional[SharedKVLayout]:
+    """Host arrays in, host tensors out.  `entry_tokens[e]` / `entry_key[e]`: length and identity (any value equal
+    for aliases of one stored shard and different otherwise: the shard's byte offset in the receive buffer will
+    do) of the K/V entries, listed task by task; the entries of task t add up to task_kv_lens[t].  Returns None
+    when the tasks of some document do not read nested prefixes of one shard sequence (then the per-task
+    unpack has to be used)."""
+    entry_tokens = [int(x) for x in entry_tokens]
+    entry_key = [int(x) for x in entry_key]
+    tasks: List[List[int]] = []
+    e = 0
+    for lk in task_kv_lens:
+        lk, got, mine = int(lk), 0, []
+        while got < lk:
+            if e >= len(entry_tokens):
+                return None
+            if entry_tokens[e] > 0:
+                mine.append(e)
+            got += entry_tokens[e]
+            e += 1
+        if got != lk:
+            return None
+        tasks.append(mine)
+    # a document = the tasks whose first entry is the same stored shard; its shard sequence = its longest task's
+    docs: dict = {}
+    order: List[int] = []
+    for t, mine in enumerate(tasks):
+        if not mine:
+            continue
+        head = entry_key[mine[0]]
+        if head not in docs:
+            docs[head] = mine
+            order.append(head)
+        elif len(mine) > len(docs[head]):
+            docs[head] = mine
+    for mine in tasks:
+        if mine:
+            ref = docs[entry_key[mine[0]]]
+            if [entry_key[x] for x in mine] != [entry_key[x] for x in ref[:len(mine)]]:
+                return None
+    first_entry: dict = {}
+    for idx, key in enumerate(entry_key):
+        if entry_tokens[idx] > 0:
+            first_entry.setdefault(key, idx)
+    store_tokens, entry_of_stored, doc_start, row = [], [], {}, 0
+    seen = set()
+    for head in order:
+        doc_start[head] = row
+        for x in docs[head]:
+            key = entry_key[x]
+            if key in seen:
+                return None   # one shard in two documents' sequences: not a prefix structure
+            seen.add(key)
+            store_tokens.append(entry_tokens[x])
+            entry_of_stored.append(first_entry[key])
+            row += entry_tokens[x]
+    offs = [doc_start[entry_key[mine[0]]] if mine else 0 for mine in tasks]
+    return SharedKVLayout(torch.tensor(store_tokens, dtype=torch.int64), torch.tensor(entry_of_stored, dtype=torch.int64),
+                          torch.tensor(offs, dtype=torch.int32), row)
+
+
+@dataclass
 class SingleRankPlan:
     """Everything one CA-server tick needs for `docs` (host tensors; `.to(device)` variants
     are built by server_metas)."""
@@ -267,10 +341,11 @@ def single_rank_plan(docs: Sequence[Sequence[int]], num_heads_q: int, num_heads_
                           entry_tokens_t, entry_shard_t, dedup, num_heads_q, num_heads_kv, head_dim, itemsize)
 
 
-def server_metas(plan: SingleRankPlan, device="cuda"):
+def server_metas(plan: SingleRankPlan, device="cuda", shared_kv: bool = True):
     """(PackedSeqParams, ServerFwdMeta, ServerBwdMeta, buffer sizes) on `device` for one tick:
-    sizes = (fwd receive, fwd send, bwd receive, bwd send) bytes."""
-    from .fused_comm_attn import ServerBwdMeta, ServerFwdMeta
+    sizes = (fwd receive, fwd send, bwd receive, bwd send) bytes.  With `shared_kv` the metas also carry the
+    layout that keeps one copy of every K/V shard (SharedKVLayout), which the in-place ticks use."""
+    from .fused_comm_attn import ServerBwdMeta, ServerFwdMeta, SharedKVOnDevice
     i64 = lambda t: _dev(t, torch.int64, device)
     attn = get_attn_metadata(plan.q_seqlens, plan.kv_seqlens, get_packed_seq_params=True)
     attn.cu_seqlens_q = _dev(attn.cu_seqlens_q, torch.int32, device)
@@ -282,12 +357,17 @@ def server_metas(plan: SingleRankPlan, device="cuda"):
     fo, _, _, f_send = plan.reply_layout(False)
     fwd = ServerFwdMeta(i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(fq), i64(fk), i64(fv),
                         i64(plan.q_seqlens), i64(fo), (tq, hq_d), (tk, hkv_d))
+    shared = shared_kv_layout(plan.kv_seqlens.tolist(), plan.kv_entry_tokens.tolist(), plan.kv_entry_shard.tolist()) if shared_kv else None
+    if shared is not None:
+        fwd.shared_kv = SharedKVOnDevice.build(shared, fk, fv, device)
     bq, bk, bv, b_recv = plan.request_layout(True)
     gq, gk, gv, b_send = plan.reply_layout(True)
     d = plan.dedup.normalize(device)
     bwd = ServerBwdMeta(i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(bq), i64(bk), i64(bv),
                         i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(gq), i64(gk), i64(gv),
                         d.main_copy_mask, d.num_copies, d.copy_start_id, (tq, hq_d), (tq, plan.num_heads_q), (tk, hkv_d))
+    if shared is not None:
+        bwd.shared_kv = SharedKVOnDevice.build(shared, bk, bv, device, gk, gv)
     return attn, fwd, bwd, (f_recv, f_send, b_recv, b_send)
 
 
@@ -309,6 +389,37 @@ class PingPangSingleStepPackedSeqParams:
     stream: object = None
     dispatcher_id: int = None
     kv_task_offsets: Optional[Tensor] = None
+    # set by to_device(): the one-copy K/V layouts of the forward and backward ticks (fused_comm_attn.SharedKVOnDevice),
+    # None when the tasks do not read nested prefixes
+    shared_kv_fwd: object = None
+    shared_kv_bwd: object = None
+
+    def _shared_kv(self, device):
+        """The SharedKVLayout of this step's tasks, from the host copies of the metadata: the K/V entries of the
+        receive side are listed task by task, aliases of a shard share their byte offset."""
+        from .fused_comm_attn import SharedKVOnDevice
+        host = lambda t: t.detach().cpu().to(torch.int64)
+        out = []
+        for req, grad, cu in ((self.qkv_fwd_metadata, None, self.cu_seqlens_kv),
+                              (self.attn_out_bwd_metadata, self.qkv_bwd_metadata,
+                               self.bwd_packed_seq_params.cu_seqlens_kv if self.bwd_packed_seq_params is not None else None)):
+            if req is None or cu is None or len(req.recv_memcpy_metadata) < 3:
+                out.append(None)
+                continue
+            k_off, v_off = host(req.recv_memcpy_metadata[1]), host(req.recv_memcpy_metadata[2])
+            if k_off.dim() != 1:
+                out.append(None)
+                continue
+            lens = host(cu).diff().tolist()
+            layout = shared_kv_layout(lens, host(req.seq_lens[1].recv_seqlens).tolist(), k_off.tolist())
+            if layout is None:
+                out.append(None)
+                continue
+            gk = gv = None
+            if grad is not None:
+                gk, gv = host(grad.send_memcpy_metadata[1]), host(grad.send_memcpy_metadata[2])
+            out.append(SharedKVOnDevice.build(layout, k_off, v_off, device, gk, gv))
+        return out
 
     def to_device(self, device="cuda"):
         to_i32 = lambda t: None if t is None else _dev(t, torch.int32, device)
@@ -317,11 +428,12 @@ class PingPangSingleStepPackedSeqParams:
         if bwd is not None:
             bwd = type(bwd)(cu_seqlens_q=to_i32(bwd.cu_seqlens_q), cu_seqlens_kv=to_i32(bwd.cu_seqlens_kv),
                             max_seqlen_q=to_int(bwd.max_seqlen_q), max_seqlen_kv=to_int(bwd.max_seqlen_kv))
+        shared_fwd, shared_bwd = self._shared_kv(device)
         return PingPangSingleStepPackedSeqParams(
             self.qkv_format, to_i32(self.cu_seqlens_q), to_i32(self.cu_seqlens_kv), to_int(self.max_seqlen_q),
             to_int(self.max_seqlen_kv), self.qkv_fwd_metadata.normalize(device), self.qkv_bwd_metadata.normalize(device),
             self.attn_out_fwd_metadata.normalize(device), self.attn_out_bwd_metadata.normalize(device), bwd, self.stream,
-            self.dispatcher_id, to_i32(self.kv_task_offsets))
+            self.dispatcher_id, to_i32(self.kv_task_offsets), shared_fwd, shared_bwd)
 
 
 def single_rank_step_params(plan: SingleRankPlan) -> PingPangSingleStepPackedSeqParams:

@@ -255,6 +255,188 @@ def test_server_tick_from_single_rank_plan(cuda):
     assert_close_bf16(tb(dv, 2), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
 
 
+def test_shared_kv_backward_tick_from_single_rank_plan(cuda):
+    """The tick that keeps ONE copy of every K/V shard (metadata.SharedKVLayout): the backward with the
+    non-deterministic switch unpacks each stored shard once, the kernels sum dK/dV over the tasks that read it, and one
+    pack writes the result: no per-task prefix copies, no duplicate-gradient sum, no mask.  dq bytes are those of the
+    step-by-step tick; dk / dv, summed in fp32 and rounded once, meet the single-kernel bar against the
+    whole-document oracle (the step-by-step tick, with one bf16 rounding per task and per summed copy, needs twice
+    that)."""
+    from distca_amd import metadata
+    from distca_amd.fused_comm_attn import FlashAttnArgs, ca_server_backward, ca_server_forward
+    docs = [[130, 257, 64, 300], [90, 10], [513]]
+    plan = metadata.single_rank_plan(docs, 8, 2)
+    fa_params, fmeta, bmeta, (f_recv, f_send, b_recv, b_send) = metadata.server_metas(plan, cuda)
+    assert fmeta.shared_kv is not None and bmeta.shared_kv is not None
+    assert bmeta.shared_kv.num_rows == plan.num_q_tokens < plan.num_kv_tokens
+    fa_args = FlashAttnArgs(8, 2, 128, deterministic=False)
+    T = plan.num_q_tokens
+    q, k, v, do = make_qkv(T, T, 8, 2, 128, 34)
+    as_bytes = lambda x: x.reshape(x.shape[0], -1).contiguous().view(torch.uint8).numpy()
+    stored = plan.stored_shard_tokens.numpy()
+    first_entry = [plan.kv_entry_shard.tolist().index(s) for s in range(len(stored))]
+    cu_doc = np.concatenate([[0], np.cumsum([sum(d) for d in docs])]).astype(np.int32)
+
+    q_off, k_off, v_off, _ = plan.request_layout(False)
+    recv = np.zeros(f_recv, np.uint8)
+    fa2a.copy_non_cp(as_bytes(q), recv, q_off.numpy(), plan.q_seqlens.numpy())
+    fa2a.copy_non_cp(as_bytes(k), recv, k_off.numpy()[first_entry], stored)
+    fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
+    send = torch.zeros(f_send, dtype=torch.uint8, device=cuda)
+    print("shared-kv forward", flush=True)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args, in_place=False)
+    torch.cuda.synchronize()
+    reply_lse = lse.T.contiguous().cpu().view(torch.uint8).numpy().reshape(T, -1)
+
+    merged = np.zeros((T, plan.merged_q_bytes), np.uint8)
+    c = 0
+    for part in (as_bytes(do), as_bytes(out.cpu()), reply_lse, as_bytes(q)):
+        merged[:, c:c + part.shape[1]] = part; c += part.shape[1]
+    q_off, k_off, v_off, _ = plan.request_layout(True)
+    recv = np.zeros(b_recv, np.uint8)
+    fa2a.copy_non_cp(merged, recv, q_off.numpy(), plan.q_seqlens.numpy())
+    fa2a.copy_non_cp(as_bytes(k), recv, k_off.numpy()[first_entry], stored)
+    fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
+    sends = []
+    for in_place in (True, False):
+        g = torch.full((b_send,), 0x3C, dtype=torch.uint8, device=cuda)
+        print(f"shared-kv backward in_place={in_place}", flush=True)
+        ca_server_backward(torch.from_numpy(recv).to(cuda), g, bmeta, fa_args, fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
+                           fa_params.max_seqlen_q, fa_params.max_seqlen_kv, in_place=in_place)
+        sends.append(g.cpu().numpy())
+    gq_off, gk_off, gv_off, _ = plan.reply_layout(True)
+    unpack = lambda g, off, lens, tb: (lambda a: (fa2a.copy_non_cp(a, g, off, lens, None, False), a)[1])(np.zeros((T, tb), np.uint8))
+    tb = lambda a, h: torch.from_numpy(a).view(torch.bfloat16).reshape(T, h, 128)
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=out.cpu().reshape(T, 8, 128), softmax_lse=lse.cpu())
+    dq = [unpack(g, gq_off.numpy(), plan.q_seqlens.numpy(), plan.q_bytes) for g in sends]
+    assert np.array_equal(dq[0], dq[1]), "dq bytes of the shared-K/V tick and of the step-by-step tick"
+    assert_close_bf16(tb(dq[0], 8), ref_dq, "dq")
+    dk = unpack(sends[0], gk_off.numpy()[first_entry], stored, plan.k_bytes)
+    dv = unpack(sends[0], gv_off.numpy()[first_entry], stored, plan.k_bytes)
+    assert_close_bf16(tb(dk, 2), ref_dk, "dk")
+    assert_close_bf16(tb(dv, 2), ref_dv, "dv")
+    # nothing but the shards' own regions was written: the bytes outside them still hold the fill
+    touched = np.zeros(b_send, bool)
+    for off, lens, tbytes in ((gq_off.numpy(), plan.q_seqlens.numpy(), plan.q_bytes), (gk_off.numpy()[first_entry], stored, plan.k_bytes),
+                              (gv_off.numpy()[first_entry], stored, plan.k_bytes)):
+        for o, n in zip(off, lens):
+            touched[o:o + n * tbytes] = True
+    assert (sends[0][~touched] == 0x3C).all()
+
+
+def test_config3_ca_tasks_as_a_server_tick(cuda):
+    """BASELINE config 3 (variant b at full size: 15 CA tasks, 262144 query rows, documents of up to 524288 tokens)
+    through the server ticks.  The receive buffer holds every document's K/V once; with the reference's layout the
+    server would have to materialise one prefix copy per task (2.4 million K/V rows here, and 17 million in variant
+    a), with the shared layout it unpacks each document once.  The reply of the forward tick and the dq part of the
+    backward reply are bit for bit what the attention entry points give on unpacked tensors with kv_task_offsets;
+    dk / dv (summed with float atomics in either form) agree to a bf16 unit in the last place."""
+    from distca_amd import metadata, workloads
+    from distca_amd.fused_comm_attn import (FlashAttnArgs, PackedSeqParams, ServerBwdMeta, ServerFwdMeta, SharedKVOnDevice,
+                                            ca_server_backward, ca_server_forward, ca_varlen_bwd, ca_varlen_fwd)
+    from distca_amd.ops import a2a_memcpy_non_cp
+    b = workloads.config3_ca_tasks(variant="b")
+    hq, hkv, d = 32, 8, 128
+    qb, kb = hq * d * 2, hkv * d * 2
+    out_tb, req_tb = qb + hq * 4, 3 * qb + hq * 4          # both multiples of 16 at 32 heads
+    nt = len(b.q_lens)
+    # every document is cut at the ends of its tasks' prefixes; a task's K/V entries are the shards up to its end
+    doc_of = {int(o): i for i, o in enumerate(sorted(set(b.kv_task_offsets.tolist())))}
+    ends = {dd: sorted({int(l) for l, o in zip(b.k_lens, b.kv_task_offsets) if doc_of[int(o)] == dd}) for dd in doc_of.values()}
+    shard_id, stored_tokens, stored_row = {}, [], []
+    for o, dd in sorted(doc_of.items()):
+        prev = 0
+        for e in ends[dd]:
+            shard_id[(dd, e)] = len(stored_tokens)
+            stored_tokens.append(e - prev); stored_row.append(o + prev); prev = e
+    entry_tokens, entry_shard = [], []
+    for l, o in zip(b.k_lens, b.kv_task_offsets):
+        dd = doc_of[int(o)]
+        for e in ends[dd]:
+            if e <= int(l):
+                entry_tokens.append(stored_tokens[shard_id[(dd, e)]]); entry_shard.append(shard_id[(dd, e)])
+    layout = metadata.shared_kv_layout(b.k_lens.tolist(), entry_tokens, entry_shard)
+    assert layout is not None and layout.num_rows == sum(stored_tokens) < sum(entry_tokens)
+    print(f"cfg3b tick: {nt} tasks, {len(stored_tokens)} stored shards ({layout.num_rows} rows), {len(entry_tokens)} entries "
+          f"({sum(entry_tokens)} rows if every task had its own copy)", flush=True)
+
+    q, k, v, do, cu_q, cu_k = _dev_inputs_cfg3(b, cuda)
+    kv_off = torch.tensor(b.kv_task_offsets, dtype=torch.int32, device=cuda)
+    mq, mk = int(max(b.q_lens)), int(max(b.k_lens))
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+    dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, kv_task_offsets=kv_off)
+
+    i64 = lambda x: torch.tensor(np.asarray(x), dtype=torch.int64, device=cuda)
+    q_lens = i64(b.q_lens)
+    st_tok = i64(stored_tokens)
+    # receive buffer of the forward tick: q tokens per task, then every stored K shard, then every stored V shard
+    q_off = i64(np.concatenate([[0], np.cumsum(b.q_lens * qb)[:-1]]))
+    kbase = int(b.q_lens.sum()) * qb
+    ks_off = kbase + np.concatenate([[0], np.cumsum(np.asarray(stored_tokens) * kb)[:-1]])
+    vs_off = ks_off + sum(stored_tokens) * kb
+    recv = torch.empty(kbase + 2 * sum(stored_tokens) * kb, dtype=torch.uint8, device=cuda)
+    # the stored shards lie in the k tensor at rows stored_row[s]: pack them shard by shard
+    src_rows = torch.cat([torch.arange(r, r + n, device=cuda) for r, n in zip(stored_row, stored_tokens)])
+    a2a_memcpy_non_cp(q.reshape(q.shape[0], -1), q_off, q_lens, True, buffer=recv)
+    a2a_memcpy_non_cp(k.reshape(k.shape[0], -1)[src_rows], i64(ks_off), st_tok, True, buffer=recv)
+    a2a_memcpy_non_cp(v.reshape(v.shape[0], -1)[src_rows], i64(vs_off), st_tok, True, buffer=recv)
+    # the store keeps documents in order of first appearance among the tasks; its row of stored shard s:
+    store_row_of_entry = {int(e): int(r) for e, r in zip(layout.entry_of_stored.tolist(),
+                                                         np.concatenate([[0], np.cumsum(layout.store_tokens.numpy())[:-1]]))}
+    e_k_off = torch.tensor([ks_off[s] for s in entry_shard], dtype=torch.int64)
+    e_v_off = torch.tensor([vs_off[s] for s in entry_shard], dtype=torch.int64)
+    out_off = i64(np.concatenate([[0], np.cumsum(b.q_lens * out_tb)[:-1]]))
+    fmeta = ServerFwdMeta(q_lens, i64(entry_tokens), q_off, e_k_off.to(cuda), e_v_off.to(cuda), q_lens, out_off,
+                          (b.total_q, hq * d), (sum(entry_tokens), hkv * d),
+                          shared_kv=SharedKVOnDevice.build(layout, e_k_off, e_v_off, cuda))
+    fa_params = PackedSeqParams(cu_q, cu_k, mq, mk)
+    fa_args = FlashAttnArgs(hq, hkv, d, deterministic=False)
+    send = torch.zeros(b.total_q * out_tb, dtype=torch.uint8, device=cuda)
+    print("cfg3b forward tick", flush=True)
+    ca_server_forward(recv, send, fmeta, fa_params, fa_args)
+    torch.cuda.synchronize()
+    tok = send.view(b.total_q, out_tb)                      # tasks' tokens are laid out in task order here
+    assert torch.equal(tok[:, :qb].contiguous().view(torch.bfloat16).view(b.total_q, hq, d), out)
+    assert torch.equal(tok[:, qb:].contiguous().view(torch.float32), lse.T.contiguous())
+
+    # backward tick: request tokens [dO | O | lse | q] per task, K/V as before; reply dq per task, dk / dv per stored shard
+    req = torch.empty((b.total_q, req_tb), dtype=torch.uint8, device=cuda)
+    for c0, part in ((0, do.reshape(b.total_q, -1)), (qb, out.reshape(b.total_q, -1)), (2 * qb, lse.T.contiguous()), (2 * qb + hq * 4, q.reshape(b.total_q, -1))):
+        pb_ = part.contiguous().view(torch.uint8).view(b.total_q, -1)
+        req[:, c0:c0 + pb_.shape[1]] = pb_
+    rq_off = i64(np.concatenate([[0], np.cumsum(b.q_lens * req_tb)[:-1]]))
+    kbase2 = b.total_q * req_tb
+    recv2 = torch.empty(kbase2 + 2 * sum(stored_tokens) * kb, dtype=torch.uint8, device=cuda)
+    recv2[:kbase2] = req.view(-1)
+    recv2[kbase2:] = recv[kbase:]
+    shift = kbase2 - kbase
+    gsend = torch.zeros(b.total_q * qb + 2 * sum(stored_tokens) * kb, dtype=torch.uint8, device=cuda)
+    gk_off = e_k_off - kbase + b.total_q * qb
+    gv_off = e_v_off - kbase + b.total_q * qb
+    bmeta = ServerBwdMeta(q_lens, i64(entry_tokens), rq_off, (e_k_off + shift).to(cuda), (e_v_off + shift).to(cuda),
+                          q_lens, i64(entry_tokens), q_off, gk_off.to(cuda), gv_off.to(cuda), None, None, None,
+                          (b.total_q, hq * d), (b.total_q, hq), (sum(entry_tokens), hkv * d),
+                          shared_kv=SharedKVOnDevice.build(layout, e_k_off + shift, e_v_off + shift, cuda, gk_off, gv_off))
+    print("cfg3b backward tick", flush=True)
+    ca_server_backward(recv2, gsend, bmeta, fa_args, cu_q, cu_k, mq, mk)
+    torch.cuda.synchronize()
+    assert torch.equal(gsend[:b.total_q * qb].view(torch.bfloat16).view(b.total_q, hq, d), dq)
+    for name, full, base in (("dk", dk, b.total_q * qb), ("dv", dv, b.total_q * qb + sum(stored_tokens) * kb)):
+        got = gsend[base:base + sum(stored_tokens) * kb].view(torch.bfloat16).view(-1, hkv, d)    # stored shards in order
+        want = full[src_rows]
+        err = ((got.float() - want.float()).abs() / want.float().abs().clamp_min(2.0 ** -6)).max().item()
+        assert err <= 2.0 ** -7, f"{name}: tick against the attention entry point {err:.2e}"
+
+
+def _dev_inputs_cfg3(batch, cuda):
+    g = torch.Generator(device=cuda).manual_seed(61)
+    rnd = lambda *shape: torch.randn(shape, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v, do = rnd(batch.total_q, 32, 128), rnd(batch.kv_rows, 8, 128), rnd(batch.kv_rows, 8, 128), rnd(batch.total_q, 32, 128)
+    cu_q = torch.tensor(batch.cu_seqlens_q, dtype=torch.int32, device=cuda)
+    cu_k = torch.tensor(batch.cu_seqlens_k, dtype=torch.int32, device=cuda)
+    return q, k, v, do, cu_q, cu_k
+
+
 def test_layer_step_with_alltoall_metadata(cuda):
     """Linear side and attention server of one layer step on one GPU (world size 1: the all-to-all
     moves nothing, send and receive buffer are the same memory), every hop through the ops of this

@@ -117,3 +117,29 @@ def test_alltoall_metadata_get_slice():
     assert r1.my_rank_send_offset == 10 and r1.my_rank_send_sz == 6
     assert r1.send_memcpy_metadata[0].tolist() == [3, 4, 5] and r1.recv_memcpy_metadata[0].tolist() == [6, 8, 10]
     assert r1.seq_lens[0].recv_seqlens.tolist() == [2, 2, 2] and r1.tensor_shape[0].recv_shape == torch.Size((6, 8))
+
+
+def test_shared_kv_layout_keeps_one_copy_per_shard_and_documents_contiguous():
+    """Tasks listed in any order; every task's prefix must be one run of store rows starting at its document."""
+    from distca_amd.metadata import shared_kv_layout
+    # documents A = shards (3, 5, 2), B = (4,), C = (6, 1); stored shard ids 0..5; tasks: (A,1) (C,0) (A,0) (B,0) (A,2) (C,1)
+    tasks = [[0, 1], [4], [0], [3], [0, 1, 2], [4, 5]]
+    tokens = {0: 3, 1: 5, 2: 2, 3: 4, 4: 6, 5: 1}
+    entry_key = [s for t in tasks for s in t]
+    entry_tokens = [tokens[s] for s in entry_key]
+    lens = [sum(tokens[s] for s in t) for t in tasks]
+    lay = shared_kv_layout(lens, entry_tokens, entry_key)
+    assert lay.num_rows == sum(tokens.values())
+    # order of first appearance of the documents: A, C, B; shards of a document in document order
+    assert lay.store_tokens.tolist() == [3, 5, 2, 6, 1, 4]
+    starts = dict(zip([0, 1, 2, 4, 5, 3], np.concatenate([[0], np.cumsum(lay.store_tokens.numpy())[:-1]]).tolist()))
+    assert lay.kv_task_offsets.tolist() == [starts[t[0]] for t in tasks]
+    assert [entry_key[e] for e in lay.entry_of_stored.tolist()] == [0, 1, 2, 4, 5, 3]
+    assert all(entry_key.index(entry_key[e]) == e for e in lay.entry_of_stored.tolist())   # the first of its aliases
+    # an empty task and zero-length entries are tolerated
+    lay = shared_kv_layout([3, 0, 8], [3, 0, 3, 5], [0, 9, 0, 1])
+    assert lay.store_tokens.tolist() == [3, 5] and lay.kv_task_offsets.tolist() == [0, 0, 0]
+    # tasks that do not read nested prefixes (the second skips shard 1): no shared layout
+    assert shared_kv_layout([8, 5], [3, 5, 3, 2], [0, 1, 0, 2]) is None
+    # entries that do not add up to the task lengths
+    assert shared_kv_layout([4], [3], [0]) is None
