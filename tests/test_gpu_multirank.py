@@ -32,15 +32,44 @@ def test_layer_step_of_several_ranks(cuda, seed, world, docs, max_shards, lo, hi
     _layer_step(cuda, world, _plan(seed, world, docs, max_shards, lo, hi), seed, replicas=True)
 
 
+def _planner_for_the_test(world, tolerance):
+    from types import SimpleNamespace
+    from distca_amd.planner import Planner
+    return Planner(world_size=world, tolerance_factor=tolerance,
+                   parallel_config=SimpleNamespace(tensor_model_parallel_size=1, pipeline_model_parallel_size=1),
+                   model_config=SimpleNamespace(hidden_size=8 * 128, num_attention_heads=8, num_key_value_heads=2))
+
+
 def test_layer_step_of_a_planned_batch(cuda):
-    """The plan comes from the planner: four ranks, one of them with a long document whose middle
-    layers are handed to the others."""
-    from distca_amd.planner import PlannerConfig, plan_cost_per_rank, plan_documents
+    """The plan comes from the planner's item surface (Item -> Planner.items_to_shardinfo): four
+    ranks, one of them with a long document whose middle layers are handed to the others."""
+    from distca_amd.planner import Item, plan_cost_per_rank
     docs = [[2600, 300], [420], [150, 90, 64], [700]]
-    plan, load = plan_documents(docs, PlannerConfig(tolerance=0.02))
-    assert plan_cost_per_rank(plan, 4) == load and max(load) < 1.1 * sum(load) / 4
+    planner = _planner_for_the_test(4, 0.02)
+    items = []
+    for r, lens in enumerate(docs):
+        for n in lens:
+            items.append(Item(planner.model_config, n, len(items), r, r, {"q": n, "kv": n}))
+    plan = planner.items_to_shardinfo(items)
+    load = plan_cost_per_rank(plan, 4)
+    assert sum(load) == sum(n * (n + 1) // 2 for lens in docs for n in lens) and max(load) < 1.1 * sum(load) / 4
     assert len(plan[0]) >= 5, "the long document is cut into nested layers"
     _layer_step(cuda, 4, plan, 14, replicas=True)
+
+
+def test_layer_step_of_a_planned_batch_whose_documents_span_ranks(cuda):
+    """Context-parallel placement (batch_to_items_general): ranks of 1024 tokens, a document of 2200
+    tokens lies on three of them as head and tail spans; the planner then balances the servers."""
+    from distca_amd.planner import batch_to_items_general, plan_cost_per_rank
+    planner = _planner_for_the_test(4, 0.05)
+    lens = [2200, 500, 372, 1024]
+    items = batch_to_items_general([lens], 1024, 4, planner.model_config)
+    assert sum(1 for it in items if it.seqid == 0) == 3
+    plan = planner.items_to_shardinfo(items)
+    assert [sum(s.shard_len for s in doc) for doc in plan] == lens and len({s.rid for s in plan[0]}) == 3
+    load = plan_cost_per_rank(plan, 4)
+    assert max(load) < 1.1 * sum(load) / 4 + 2201
+    _layer_step(cuda, 4, plan, 16, replicas=True)
 
 
 def test_layer_step_with_an_idle_server_and_an_empty_owner(cuda):
