@@ -18,7 +18,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .ops import a2a_memcpy_non_cp, a2a_memcpy_non_cp_multi, pre_a2a_grad_acc
+from .ops import DispatcherWrapper, a2a_memcpy_non_cp, a2a_memcpy_non_cp_multi, pre_a2a_grad_acc
 from .utils import size_pad_by_int4
 from .dispatch import (post_a2a_attn_out, post_a2a_attn_out_grad_resend_qkv, post_a2a_qkv, pre_a2a_attn_out_grad_resend_qkv,
                        pre_a2a_attn_out_with_lse, pre_a2a_qkv)
@@ -471,14 +471,90 @@ def fused_comm_attn_backward(recv_buffer: Tensor, send_buffer: Tensor, packed_se
                               bwd.max_seqlen_q, bwd.max_seqlen_kv, dtype)
 
 
-def post_a2a_attn_out_with_lse(recv_buffer: Tensor, q: Tensor, num_heads_q: int, metadata, dtype: torch.dtype = None):
+def _server_buffers(dispatcher_id):
+    """(receive buffer, send buffer) of one tick through the dispatcher, with the reference's
+    bookkeeping (dispatch.py:60-94 of the reference, then :97-106): the receive buffer is the named
+    instance's, or the current one's, which then stops being current; the reply goes into the
+    instance that is named, or current after that switch.  The caller releases a named instance
+    once its kernels are enqueued (`_server_done`)."""
+    if dispatcher_id is not None:
+        assert DispatcherWrapper.is_acquired[dispatcher_id], "no all-to-all has filled this dispatcher's receive buffer"
+    recv = DispatcherWrapper.get_instance(dispatcher_id).recv_buffer
+    if dispatcher_id is None:
+        DispatcherWrapper.switch_buffer()
+    return recv, DispatcherWrapper.get_instance(dispatcher_id).send_buffer
+
+
+def _server_done(dispatcher_id):
+    # in-place ticks read the receive buffer from inside the attention kernels, so the release
+    # follows them in stream order rather than the unpack, as it does in the reference
+    if dispatcher_id is not None:
+        DispatcherWrapper.release(dispatcher_id)
+
+
+class FusedCommAttn(torch.autograd.Function):
+    """The CA server's tick as the reference's autograd function (fused_comm_attn.py:282-461), same
+    arguments in the same order: unpack what the q/k/v all-to-all delivered, attention, pack the
+    [out | lse] reply; its backward unpacks the request [dO | O | lse | q] + k + v, runs the attention
+    backward and packs dq and the k / v gradients of the main copies.  Tensors travel through the
+    `DispatcherWrapper` instance `dispatcher_id`; what autograd sees is a one-element signal."""
+
+    @staticmethod
+    def forward(ctx, signal: Tensor, fwd_qkv_metadata, bwd_qkv_metadata, fwd_attn_out_metadata, bwd_attn_out_qkv_metadata,
+                fwd_fa_params, bwd_fa_params, dispatcher_id: int, flash_attn_args: FlashAttnArgs):
+        qkv, out = fwd_qkv_metadata, fwd_attn_out_metadata
+        q_off, k_off, v_off = qkv.recv_memcpy_metadata
+        meta = ServerFwdMeta(qkv.seq_lens[0].recv_seqlens, qkv.seq_lens[1].recv_seqlens, q_off, k_off, v_off,
+                             out.seq_lens[0].send_seqlens, out.send_memcpy_metadata[0],
+                             tuple(qkv.tensor_shape[0].recv_shape), tuple(qkv.tensor_shape[1].recv_shape),
+                             shared_kv=getattr(fwd_fa_params, "shared_kv_fwd", None))
+        recv_buffer, send_buffer = _server_buffers(dispatcher_id)
+        ca_server_forward(recv_buffer, send_buffer, meta, fwd_fa_params, flash_attn_args, signal.dtype)
+        _server_done(dispatcher_id)
+
+        req, grad = bwd_attn_out_qkv_metadata, bwd_qkv_metadata
+        dedup = grad.kv_grad_send_dedup
+        ctx.save_for_backward(
+            req.seq_lens[0].recv_seqlens, req.seq_lens[1].recv_seqlens, *req.recv_memcpy_metadata,
+            grad.seq_lens[0].send_seqlens, grad.seq_lens[1].send_seqlens, *grad.send_memcpy_metadata,
+            dedup.main_copy_mask, dedup.num_copies, dedup.copy_start_id,
+            bwd_fa_params.cu_seqlens_q, bwd_fa_params.cu_seqlens_kv)
+        ctx.dispatcher_id = dispatcher_id
+        ctx.fa_args = flash_attn_args
+        ctx.bwd_attn_max_seqlen_q = bwd_fa_params.max_seqlen_q
+        ctx.bwd_attn_max_seqlen_kv = bwd_fa_params.max_seqlen_kv
+        tq = int(req.tensor_shape[0].recv_shape[0])
+        ctx.bwd_q_shape = (tq, flash_attn_args.num_heads_q * flash_attn_args.head_dim)
+        ctx.softmax_lse_shape = (tq, flash_attn_args.num_heads_q)
+        ctx.bwd_k_shape = tuple(req.tensor_shape[1].recv_shape)
+        ctx.shared_kv_bwd = getattr(fwd_fa_params, "shared_kv_bwd", None)
+        return torch.empty((1,), device=signal.device, dtype=signal.dtype)
+
+    @staticmethod
+    def backward(ctx, signal_grad: Tensor):
+        (q_tokens, k_tokens, q_off, k_off, v_off, gq_tokens, gk_tokens, gq_off, gk_off, gv_off,
+         main_copy_mask, num_copies, copy_start_id, cu_q, cu_kv) = ctx.saved_tensors
+        meta = ServerBwdMeta(q_tokens, k_tokens, q_off, k_off, v_off, gq_tokens, gk_tokens, gq_off, gk_off, gv_off,
+                             main_copy_mask, num_copies, copy_start_id, ctx.bwd_q_shape, ctx.softmax_lse_shape,
+                             ctx.bwd_k_shape, shared_kv=ctx.shared_kv_bwd)
+        recv_buffer, send_buffer = _server_buffers(ctx.dispatcher_id)
+        ca_server_backward(recv_buffer, send_buffer, meta, ctx.fa_args, cu_q, cu_kv, ctx.bwd_attn_max_seqlen_q,
+                           ctx.bwd_attn_max_seqlen_kv, signal_grad.dtype)
+        _server_done(ctx.dispatcher_id)
+        return (torch.empty((1,), device=signal_grad.device, dtype=signal_grad.dtype),) + (None,) * 8
+
+
+def post_a2a_attn_out_with_lse(recv_buffer: Optional[Tensor], q: Tensor, num_heads_q: int, metadata, dtype: torch.dtype = None,
+                               instance_id: int = None, switch_buffer: bool = False):
     """Linear side, forward of the reference's autograd function of the same name
     (fused_comm_attn.py:468-506): unpack the [out | lse | pad] tokens of the reply and split them.
-    Returns (attn_out [T, 1, Hq*D] in q's dtype, softmax_lse_bytes [T, Hq*4] uint8)."""
+    Returns (attn_out [T, 1, Hq*D] in q's dtype, softmax_lse_bytes [T, Hq*4] uint8).  `recv_buffer`
+    None reads the receive buffer of dispatcher instance `instance_id`."""
     dtype = dtype or q.dtype
     recv_shape = tuple(metadata.tensor_shape[0].recv_shape)    # in elements of `dtype`, as the reference has it
-    recv = torch.empty(recv_shape, dtype=dtype, device=recv_buffer.device).view(torch.uint8)
-    post_a2a_attn_out(recv, metadata.seq_lens[0].recv_seqlens, *metadata.recv_memcpy_metadata, buffer=recv_buffer)
+    recv = torch.empty(recv_shape, dtype=dtype, device=q.device).view(torch.uint8)
+    post_a2a_attn_out(recv, metadata.seq_lens[0].recv_seqlens, *metadata.recv_memcpy_metadata, switch_buffer=switch_buffer,
+                      instance_id=instance_id, buffer=recv_buffer)
     itemsize = torch.empty((), dtype=dtype).element_size()
     hidden_bytes = math.prod(q.shape[1:]) * itemsize
     lse_bytes = num_heads_q * 4
@@ -487,12 +563,14 @@ def post_a2a_attn_out_with_lse(recv_buffer: Tensor, q: Tensor, num_heads_q: int,
     return attn_out, softmax_lse_bytes
 
 
-def post_a2a_attn_out_with_lse_backward(send_buffer: Tensor, grad_attn_out: Tensor, attn_out: Tensor, softmax_lse_bytes: Tensor,
-                                        q: Tensor, k: Tensor, v: Tensor, bwd_attn_out_qkv_metadata):
+def post_a2a_attn_out_with_lse_backward(send_buffer: Optional[Tensor], grad_attn_out: Tensor, attn_out: Tensor, softmax_lse_bytes: Tensor,
+                                        q: Tensor, k: Tensor, v: Tensor, bwd_attn_out_qkv_metadata, instance_id: int = None):
     """Linear side, backward of the same function (fused_comm_attn.py:508-526): pack the request
-    [dO | O | lse | q | pad] and the K/V shards for the attention server."""
+    [dO | O | lse | q | pad] and the K/V shards for the attention server (`send_buffer` None: into the
+    send buffer of dispatcher instance `instance_id`)."""
     flat = lambda t: t.reshape(t.shape[0], math.prod(t.shape[1:]))   # -1 is ambiguous for a rank that holds no tokens
     md = bwd_attn_out_qkv_metadata
     pre_a2a_attn_out_grad_resend_qkv(
         flat(grad_attn_out), flat(attn_out), softmax_lse_bytes, flat(q), flat(k), flat(v), md.kv_replica_mask,
-        md.seq_lens[0].send_seqlens, md.seq_lens[1].send_seqlens, *md.send_memcpy_metadata, buffer=send_buffer)
+        md.seq_lens[0].send_seqlens, md.seq_lens[1].send_seqlens, *md.send_memcpy_metadata,
+        instance_id=instance_id, buffer=send_buffer)

@@ -2,14 +2,15 @@
 
 Same names, argument order and error behaviour as the reference's Python wrappers
 (distca/runtime/attn_kernels/ops.py:153-215), bound to the HIP kernels through the C ABI
-instead of torch.ops.dispatch_kernels.  The reference can take its transport buffer from
-an NVSHMEM dispatcher; here the buffer is always an explicit device tensor (the
-reference's `buffer=` form, csrc/bindings/all_to_all.cpp:102-113,243-254): on one GPU a
-task buffer is ordinary device memory.
+instead of torch.ops.dispatch_kernels.  The transport buffer is either an explicit device
+tensor (the reference's `buffer=` form, csrc/bindings/all_to_all.cpp:102-113,243-254) or, as
+in the reference's normal mode, the send / receive buffer of the `DispatcherWrapper` instance
+`instance_id` names.  The transport between ranks is not part of this package: the
+dispatcher's buffers are ordinary device memory and `fast_a2a` covers a world of one rank.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import List, Optional
 
 import torch
 
@@ -38,6 +39,91 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+class DispatcherWrapper:
+    """Who owns the transport buffers (distca/runtime/attn_kernels/ops.py:67-150).  Two instances,
+    for the two halves of a ping-pong step; each holds a send and a receive buffer of
+    `buffer_size` bytes.  `acquire` / `release` keep the reference's bookkeeping (a receive buffer
+    is acquired by the all-to-all that fills it and released by the op that has unpacked it, and
+    the memcpy ops check that order) without the cross-rank signal behind it."""
+    instance: Optional[List["DispatcherWrapper"]] = None
+    is_acquired: List[bool] = [False, False]
+    cur_instance: int = 0
+
+    def __init__(self, buffer_size: int, device):
+        self.buffer_size = int(buffer_size)
+        self.device = torch.device(device)
+        self.send_buffer = torch.zeros(self.buffer_size, dtype=torch.uint8, device=self.device)
+        self.recv_buffer = torch.zeros(self.buffer_size, dtype=torch.uint8, device=self.device)
+
+    @staticmethod
+    def init(rank: int = 0, local_rank: int = 0, world_size: int = 1, buffer_size: int = 0, uid=None, device="cuda"):
+        if world_size != 1:
+            raise NotImplementedError("the transport between ranks is not part of this package: world_size must be 1")
+        DispatcherWrapper.instance = [DispatcherWrapper(buffer_size, device) for _ in range(2)]
+        DispatcherWrapper.is_acquired = [False, False]
+        DispatcherWrapper.cur_instance = 0
+
+    @staticmethod
+    def get_instance(instance_id: Optional[int] = None) -> "DispatcherWrapper":
+        if DispatcherWrapper.instance is None:
+            raise AssertionError("DispatcherWrapper not initialized")
+        return DispatcherWrapper.instance[DispatcherWrapper.cur_instance if instance_id is None else instance_id]
+
+    @staticmethod
+    def switch_buffer():
+        DispatcherWrapper.cur_instance = (DispatcherWrapper.cur_instance + 1) % 2
+
+    @staticmethod
+    def update_buffer_size(buffer_size: int):
+        """Grow both instances to `buffer_size` bytes; contents are not kept."""
+        torch.cuda.synchronize()
+        for i, inst in enumerate(DispatcherWrapper.instance):
+            assert not DispatcherWrapper.is_acquired[i]
+            if inst.buffer_size < buffer_size:
+                DispatcherWrapper.instance[i] = DispatcherWrapper(buffer_size, inst.device)
+
+    @staticmethod
+    def acquire(instance_id: int):
+        assert not DispatcherWrapper.is_acquired[instance_id]
+        DispatcherWrapper.is_acquired[instance_id] = True
+
+    @staticmethod
+    def release(instance_id: int):
+        assert DispatcherWrapper.is_acquired[instance_id]
+        DispatcherWrapper.is_acquired[instance_id] = False
+
+
+def _transport_buffer(buffer: Optional[torch.Tensor], instance_id: Optional[int], to_nvshmem: bool) -> torch.Tensor:
+    """The explicit buffer, or the dispatcher's (ops.py:160-181 of the reference: with an instance
+    id, packing needs the instance released and unpacking needs it acquired)."""
+    if buffer is not None:
+        return buffer
+    if instance_id is not None:
+        if to_nvshmem:
+            assert not DispatcherWrapper.is_acquired[instance_id], "pack into a dispatcher whose receive buffer is not released"
+        else:
+            assert DispatcherWrapper.is_acquired[instance_id], "unpack from a dispatcher no all-to-all has filled"
+    inst = DispatcherWrapper.get_instance(instance_id)
+    return inst.send_buffer if to_nvshmem else inst.recv_buffer
+
+
+def fast_a2a(sender_send_disp: torch.Tensor, sender_transfer_sz: torch.Tensor, sender_recv_disp: torch.Tensor,
+             recver_transfer_sz: torch.Tensor, my_rank_send_offset: int, my_rank_recv_offset: int, my_rank_send_sz: int,
+             instance_id: Optional[int] = None):
+    """The all-to-all of a world of one rank (ops.py:217-262 of the reference): what a rank sends to
+    itself goes from the send buffer to the receive buffer as one device copy, and the receive buffer
+    counts as acquired from then on.  More ranks need a transport, which this package does not hold."""
+    if sender_send_disp.numel() != 1:
+        raise NotImplementedError("fast_a2a: the transport between ranks is not part of this package")
+    if instance_id is not None:
+        DispatcherWrapper.acquire(instance_id)
+    inst = DispatcherWrapper.get_instance(instance_id)
+    n = int(my_rank_send_sz)
+    if my_rank_send_offset + n > inst.buffer_size or my_rank_recv_offset + n > inst.buffer_size:
+        raise RuntimeError(f"fast_a2a: {n} bytes do not fit the dispatcher's buffers of {inst.buffer_size} bytes")
+    inst.recv_buffer[my_rank_recv_offset:my_rank_recv_offset + n].copy_(inst.send_buffer[my_rank_send_offset:my_rank_send_offset + n])
+
+
 def a2a_memcpy_non_cp(
     tensor: torch.Tensor, nvshmem_offset: torch.Tensor,
     shard_tokens: torch.Tensor, to_nvshmem: bool,
@@ -49,8 +135,9 @@ def a2a_memcpy_non_cp(
     Shard s covers rows excl_cumsum(shard_tokens)[s].. and buffer bytes nvshmem_offset[s]..
     `shard_do_copy_mask` (int8, packing only) skips shards whose entry is 0.
     """
-    if buffer is None:
-        raise RuntimeError("a2a_memcpy_non_cp: this build has no NVSHMEM dispatcher; pass buffer=")
+    if shard_do_copy_mask is not None and buffer is None:
+        assert to_nvshmem
+    buffer = _transport_buffer(buffer, instance_id, to_nvshmem)
     _check_tensor(2, tensor, "tensor")
     _check_tensor(1, nvshmem_offset, "seq_nvshmem_offset")
     _check_dtype(nvshmem_offset, torch.int64, "seq_nvshmem_offset")
@@ -75,7 +162,7 @@ def a2a_memcpy_non_cp(
 
 
 def a2a_memcpy_non_cp_multi(tensors, nvshmem_offsets, shard_tokens, to_nvshmem: bool, shard_do_copy_masks=None, *,
-                            buffer: torch.Tensor):
+                            buffer: Optional[torch.Tensor] = None, instance_id: Optional[int] = None):
     """Several a2a_memcpy_non_cp calls against one buffer as a single launch: tensors[i] with nvshmem_offsets[i],
     shard_tokens[i] and (packing only) shard_do_copy_masks[i].  What the reference does with consecutive calls for
     the q, k and v of a tick (distca/runtime/attn_kernels/dispatch.py:39-56,60-94); the result is the same bytes."""
@@ -86,6 +173,7 @@ def a2a_memcpy_non_cp_multi(tensors, nvshmem_offsets, shard_tokens, to_nvshmem: 
         raise RuntimeError(f"a2a_memcpy_non_cp_multi: at most {_lib.PACK_MAX_JOBS} tensors per launch")
     if n == 0:
         return None
+    buffer = _transport_buffer(buffer, instance_id, to_nvshmem)
     if not buffer.is_cuda:
         raise RuntimeError("tensor buffer must be on CUDA")
     jobs = (_lib.PackJob * n)()
@@ -120,8 +208,7 @@ def a2a_memcpy_cp(
 ):
     """Replicating pack of `tensor` [T, hidden] to every live (shard, replica) slot of
     `buffer`, or unpack into `tensor` [max_cp, T, hidden] (which the caller pre-zeroes)."""
-    if buffer is None:
-        raise RuntimeError("a2a_memcpy_cp: this build has no NVSHMEM dispatcher; pass buffer=")
+    buffer = _transport_buffer(buffer, instance_id, to_nvshmem)
     _check_tensor(2 if to_nvshmem else 3, tensor, "tensor")
     if nvshmem_offset.dim() != 2:
         raise RuntimeError("tensor seq_nvshmem_offset must have 2 dimensions")

@@ -155,8 +155,32 @@ def test_python_wrappers_reject_wrong_inputs():
     from distca_amd.fused_comm_attn import ca_varlen_fwd
     t = torch.zeros((4, 8), dtype=torch.bfloat16)
     off = torch.zeros(1, dtype=torch.int64)
-    with pytest.raises(RuntimeError, match="buffer"):
+    with pytest.raises(AssertionError, match="DispatcherWrapper not initialized"):   # ops.py:112-115 of the reference
         ops.a2a_memcpy_non_cp(t, off, off, True)
+    with pytest.raises(NotImplementedError):
+        ops.DispatcherWrapper.init(0, 0, 2, 1024, device="cpu")
+    ops.DispatcherWrapper.init(0, 0, 1, 1024, device="cpu")
+    try:
+        with pytest.raises(AssertionError, match="no all-to-all has filled"):
+            ops.a2a_memcpy_non_cp(t, off, off, False, instance_id=0)
+        ops.DispatcherWrapper.acquire(0)
+        with pytest.raises(AssertionError, match="not released"):
+            ops.a2a_memcpy_non_cp(t, off, off, True, instance_id=0)
+        ops.DispatcherWrapper.release(0)
+        ops.DispatcherWrapper.get_instance(0).send_buffer[:8] = torch.arange(8, dtype=torch.uint8)
+        one = torch.ones((1, 1), dtype=torch.int64)
+        ops.fast_a2a(one, one, one, one, 0, 16, 8, instance_id=0)
+        assert ops.DispatcherWrapper.is_acquired[0]
+        assert ops.DispatcherWrapper.get_instance(0).recv_buffer[16:24].tolist() == list(range(8))
+        with pytest.raises(RuntimeError, match="do not fit"):
+            ops.fast_a2a(one, one, one, one, 0, 1020, 8)
+        assert ops.DispatcherWrapper.get_instance() is ops.DispatcherWrapper.instance[0]
+        ops.DispatcherWrapper.switch_buffer()
+        assert ops.DispatcherWrapper.get_instance() is ops.DispatcherWrapper.instance[1]
+    finally:
+        ops.DispatcherWrapper.instance = None
+        ops.DispatcherWrapper.is_acquired = [False, False]
+        ops.DispatcherWrapper.cur_instance = 0
     with pytest.raises(RuntimeError):
         ops.a2a_memcpy_non_cp(t, off.to(torch.int32), off, True, buffer=torch.zeros(64, dtype=torch.uint8))
     with pytest.raises(RuntimeError):

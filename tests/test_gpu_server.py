@@ -492,3 +492,89 @@ def test_layer_step_with_alltoall_metadata(cuda):
     # up to three per-task bf16 gradients summed in bf16 per stored shard: 4e-2 / 3e-3
     assert_close_bf16(dk_planes.sum(0).reshape(T, hkv, d), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
     assert_close_bf16(dv_planes.sum(0).reshape(T, hkv, d), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
+
+
+def test_fused_comm_attn_autograd_function(cuda):
+    """FusedCommAttn with the reference's call (fused_comm_attn.py:282-461): `.apply(signal, four metadata
+    objects, forward and backward attention parameters, dispatcher id, FlashAttnArgs)` returns a one-element
+    signal, and `.backward()` on it runs the server's backward tick.  Tensors travel through dispatcher
+    instance 1: the linear side packs into its send buffer, the all-to-all of a one-rank world copies it to
+    the receive buffer, the server answers into the send buffer.  Forward reply and gradients are held
+    against the whole-document oracle, and, bit for bit, against the same tick on explicit buffers."""
+    from distca_amd import metadata
+    from distca_amd.dispatch import post_a2a_qkv, pre_a2a_qkv
+    from distca_amd.fused_comm_attn import (FlashAttnArgs, FusedCommAttn, fused_comm_attn_backward, fused_comm_attn_forward,
+                                            post_a2a_attn_out_with_lse, post_a2a_attn_out_with_lse_backward)
+    from distca_amd.ops import DispatcherWrapper, fast_a2a
+    docs = [[200, 56, 310], [129], [64, 64]]
+    hq, hkv, d = 8, 2, 128
+    plan = metadata.single_rank_plan(docs, hq, hkv)
+    step = metadata.single_rank_step_params(plan).to_device(cuda)
+    fa_args = FlashAttnArgs(hq, hkv, d)
+    T = plan.num_q_tokens
+    q, k, v, do = make_qkv(T, T, hq, hkv, d, 45)
+    qd, kd, vd, dod = (x.reshape(x.shape[0], -1).to(cuda) for x in (q, k, v, do))
+    mds = (step.qkv_fwd_metadata, step.qkv_bwd_metadata, step.attn_out_fwd_metadata, step.attn_out_bwd_metadata)
+    DispatcherWrapper.init(0, 0, 1, max(int(m.my_rank_send_sz) for m in mds), device=cuda)
+    ID = 1
+
+    def a2a(md):
+        fast_a2a(*md.fa2a_metadata, md.my_rank_send_offset, md.my_rank_recv_offset, md.my_rank_send_sz, instance_id=ID)
+
+    recv_of = lambda: DispatcherWrapper.get_instance(ID).recv_buffer
+    send_of = lambda: DispatcherWrapper.get_instance(ID).send_buffer
+
+    # forward
+    fwd, out_md, req, grad = step.qkv_fwd_metadata, step.attn_out_fwd_metadata, step.attn_out_bwd_metadata, step.qkv_bwd_metadata
+    pre_a2a_qkv(qd, kd, vd, fwd.kv_replica_mask, fwd.seq_lens[0].send_seqlens, fwd.seq_lens[1].send_seqlens,
+                *fwd.send_memcpy_metadata, is_fwd=True, instance_id=ID)
+    a2a(fwd)
+    assert DispatcherWrapper.is_acquired[ID]
+    explicit_reply = torch.zeros(int(out_md.my_rank_send_sz), dtype=torch.uint8, device=cuda)
+    fused_comm_attn_forward(recv_of().clone(), explicit_reply, step, fa_args)
+    signal = torch.empty((1,), dtype=torch.bfloat16, device=cuda, requires_grad=True)
+    print("FusedCommAttn.apply", flush=True)
+    out_signal = FusedCommAttn.apply(signal, fwd, grad, out_md, req, step, step.bwd_packed_seq_params, ID, fa_args)
+    assert out_signal.shape == (1,) and out_signal.dtype == torch.bfloat16 and out_signal.requires_grad
+    assert not DispatcherWrapper.is_acquired[ID], "the server has released the receive buffer"
+    n = int(out_md.my_rank_send_sz)
+    assert torch.equal(send_of()[:n], explicit_reply), "reply bytes of the autograd function and of the tick on explicit buffers"
+    a2a(out_md)
+    attn_out, lse_bytes = post_a2a_attn_out_with_lse(None, qd, hq, out_md, instance_id=ID)
+    torch.cuda.synchronize()
+    cu_doc = np.concatenate([[0], np.cumsum([sum(x) for x in docs])]).astype(np.int32)
+    ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_doc, cu_doc)
+    assert_close_bf16(attn_out.reshape(T, hq, d), ref_out, "out")
+    lse = lse_bytes.contiguous().view(torch.float32)
+    assert (lse.T.cpu() - ref_lse).abs().max().item() <= 2e-3
+
+    # backward: the linear side sends the request, then autograd drives the server
+    post_a2a_attn_out_with_lse_backward(None, dod, attn_out, lse_bytes.contiguous(), qd, kd, vd, req, instance_id=ID)
+    a2a(req)
+    explicit_grads = torch.zeros(int(grad.my_rank_send_sz), dtype=torch.uint8, device=cuda)
+    fused_comm_attn_backward(recv_of().clone(), explicit_grads, step, fa_args)
+    print("FusedCommAttn backward", flush=True)
+    out_signal.backward(torch.empty((1,), dtype=torch.bfloat16, device=cuda))
+    assert signal.grad is not None and signal.grad.shape == (1,)
+    assert not DispatcherWrapper.is_acquired[ID]
+    n = int(grad.my_rank_send_sz)
+    assert torch.equal(send_of()[:n], explicit_grads), "gradient bytes of the autograd function and of the tick on explicit buffers"
+    a2a(grad)
+    dq = torch.zeros_like(qd)
+    dk_planes = torch.zeros((1,) + tuple(kd.shape), dtype=kd.dtype, device=cuda)
+    dv_planes = torch.zeros_like(dk_planes)
+    post_a2a_qkv(dq, dk_planes, dv_planes, grad.kv_replica_mask, grad.seq_lens[0].recv_seqlens, grad.seq_lens[1].recv_seqlens,
+                 *grad.recv_memcpy_metadata, is_fwd=False, switch_buffer=False, instance_id=ID)
+    torch.cuda.synchronize()
+    ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=attn_out.cpu().reshape(T, hq, d),
+                                              softmax_lse=lse.T.contiguous().cpu())
+    assert_close_bf16(dq.reshape(T, hq, d), ref_dq, "dq")
+    assert_close_bf16(dk_planes.sum(0).reshape(T, hkv, d), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
+    assert_close_bf16(dv_planes.sum(0).reshape(T, hkv, d), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
+    # without an instance id the ticks alternate between the two instances
+    DispatcherWrapper.cur_instance = 0
+    from distca_amd.fused_comm_attn import _server_buffers
+    r0, s1 = _server_buffers(None)
+    assert r0.data_ptr() == DispatcherWrapper.instance[0].recv_buffer.data_ptr()
+    assert s1.data_ptr() == DispatcherWrapper.instance[1].send_buffer.data_ptr() and DispatcherWrapper.cur_instance == 1
+    DispatcherWrapper.instance = None
