@@ -10,7 +10,7 @@ to stderr.
 
 Algorithmic work: causal pairs P = sum_tasks [Lq*Lk - Lq(Lq-1)/2]; forward 4*Hq*D*P FLOP,
 backward 10*Hq*D*P FLOP.  `roofline` describes the dominant kernels, the two that make up the
-attention backward (ca_bwd_dkdv_kernel over key blocks, ca_bwd_dq_kernel over query blocks):
+attention backward (ca_bwd_dkdv64_kernel over key blocks, ca_bwd_dq_kernel over query blocks):
 algorithmic backward FLOPs over the sum of their launch durations, measured live by HIP events
 the library records on the launch stream.  Both recompute S and dP, so together they execute
 14*Hq*D*P FLOP for 10*Hq*D*P of algorithmic work; `executed_tflops` reports that rate per kernel.
@@ -34,8 +34,8 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
-# WRITE_SIZE (x1.000), factors from the pack kernel's known copy size in the same run
-MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.92e9, "ca_bwd_dkdv_kernel": 35.18e9, "ca_bwd_dq_kernel": 12.72e9}
+# WRITE_SIZE (x1.000), factors from the pack kernels' known copy sizes in the same run
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.95e9, "ca_bwd_dkdv64_kernel": 36.05e9, "ca_bwd_dq_kernel": 12.80e9}
 
 
 def log(*a):
@@ -168,6 +168,70 @@ def pack_unpack_bench(torch, dev, iters: int = 10):
     return res
 
 
+def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 3, shard_cap: int = 4096):
+    """The CA server's ticks on the bench workload: every document cut into shards of at most `shard_cap`
+    tokens, one CA task per shard reading its document's prefix.  Forward tick = unpack K/V (each stored shard
+    once) + attention reading q from the receive buffer and writing [out | lse] tokens into the send buffer;
+    backward tick = unpack K/V + attention backward reading [dO | O | lse | q] tokens from the receive buffer,
+    writing dq into the send buffer + pack of dk / dv.  Same causal pairs as the attention step above, so the
+    tick times compare directly with the kernel times."""
+    from distca_amd import metadata
+    from distca_amd.dispatch import TokenLayout
+    from distca_amd.fused_comm_attn import FlashAttnArgs, ca_server_backward, ca_server_forward
+    from distca_amd.ops import a2a_memcpy_non_cp_multi
+    hq, hkv, d = batch.num_heads_q, batch.num_heads_kv, batch.head_dim
+    docs = [[min(shard_cap, n - a) for a in range(0, n, shard_cap)] for n in (int(x) for x in batch.q_lens)]
+    plan = metadata.single_rank_plan(docs, hq, hkv, d)
+    fa_params, fmeta, bmeta, (f_recv, f_send, b_recv, b_send) = metadata.server_metas(plan, dev)
+    T = plan.num_q_tokens
+    flat = lambda x: x.reshape(T, -1)
+    i64 = lambda t: t.to(device=dev, dtype=torch.int64)
+    stored = i64(plan.stored_shard_tokens)
+    first_entry = {}
+    for e, s in enumerate(plan.kv_entry_shard.tolist()):
+        first_entry.setdefault(s, e)
+    first = torch.tensor([first_entry[s] for s in range(len(first_entry))], dtype=torch.int64)
+
+    def fill(recv, q_rows, backward):
+        q_off, k_off, v_off, _ = plan.request_layout(backward)
+        a2a_memcpy_non_cp_multi([q_rows, flat(k), flat(v)], [i64(q_off), i64(k_off[first]), i64(v_off[first])],
+                                [i64(plan.q_seqlens), stored, stored], True, buffer=recv)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    recv = torch.zeros(f_recv, dtype=torch.uint8, device=dev)
+    send = torch.zeros(f_send, dtype=torch.uint8, device=dev)
+    fill(recv, flat(q), False)
+    res = {"tasks": int(plan.q_seqlens.numel()), "documents": len(docs), "shard_cap": shard_cap,
+           "stored_kv_rows": T, "kv_rows_one_copy_per_task": plan.num_kv_tokens}
+    fa_det, fa_sum = FlashAttnArgs(hq, hkv, d, deterministic=True), FlashAttnArgs(hq, hkv, d, deterministic=False)
+    res["forward_ms"] = round(timed(lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det)), 3)
+    out, lse = ca_server_forward(recv, send, fmeta, fa_params, fa_det, in_place=False)
+    del recv, send
+    request = TokenLayout.of([flat(do), out, lse.T.contiguous(), flat(q)]).merge([flat(do), out, lse.T.contiguous(), flat(q)])
+    del out, lse
+    recv = torch.zeros(b_recv, dtype=torch.uint8, device=dev)
+    fill(recv, request, True)
+    del request
+    send = torch.zeros(b_send, dtype=torch.uint8, device=dev)
+    bwd = lambda fa: ca_server_backward(recv, send, bmeta, fa, fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
+                                        fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
+    res["backward_ms"] = round(timed(lambda: bwd(fa_sum)), 3)
+    res["backward_deterministic_ms"] = round(timed(lambda: bwd(fa_det)), 3)
+    res["note"] = ("backward_ms: one stored copy per K/V shard, dk / dv summed over tasks by float atomics; "
+                   "backward_deterministic_ms: one K/V prefix copy per task, duplicate gradients summed in copy order")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -176,6 +240,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU-baseline leg (0 disables)")
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--no-pack", action="store_true")
+    ap.add_argument("--no-tick", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the CA-server path; --gpus must be 1 "
@@ -249,6 +314,12 @@ def main():
             sep = pack[key]["as_separate_launches"]
             log(f"  {key:17s} as three launches {sep['GB/s']} GB/s ({100 * sep['frac_hbm_peak']:.1f}%)")
 
+    tick = None
+    if not args.no_tick:
+        tick = server_tick_bench(torch, dev, batch, q, k, v, do)
+        log(f"  server tick over {tick['tasks']} tasks: forward {tick['forward_ms']} ms, backward {tick['backward_ms']} ms "
+            f"(deterministic {tick['backward_deterministic_ms']} ms)")
+
     cpu = None
     if args.cpu_seconds > 0:
         cpu = cpu_baseline(batch, args.cpu_seconds, 77)
@@ -263,17 +334,18 @@ def main():
                                f"{tq} packed tokens, 32q/8kv heads, d=128, causal, fwd+bwd",
                    "causal_pairs": batch.causal_pairs, "flop_fwd": flop_fwd, "flop_bwd": flop_bwd,
                    "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2)},
-        "roofline": {"bound": "mfma", "kernel": "ca_bwd_dkdv_kernel + ca_bwd_dq_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "ca_bwd_dkdv64_kernel + ca_bwd_dq_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(bwd_tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": (MEASURED_TRAFFIC_BYTES["ca_bwd_dkdv_kernel"] + MEASURED_TRAFFIC_BYTES["ca_bwd_dq_kernel"]) if default_workload else None,
+                     "traffic": (MEASURED_TRAFFIC_BYTES["ca_bwd_dkdv64_kernel"] + MEASURED_TRAFFIC_BYTES["ca_bwd_dq_kernel"]) if default_workload else None,
                      "traffic_unit": "bytes per launch (both kernels)",
-                     "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv_kernel": round(dkdv_k, 4), "ca_bwd_dq_kernel": round(dq_k, 4)},
-                     "executed_tflops": {"ca_bwd_dkdv_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
+                     "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv64_kernel": round(dkdv_k, 4), "ca_bwd_dq_kernel": round(dq_k, 4)},
+                     "executed_tflops": {"ca_bwd_dkdv64_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
                      "launches": bwd_n,
                      "also": {"ca_fwd_kernel": {"achieved": round(fwd_tf, 2), "frac": round(fwd_tf / PEAK_BF16_TFLOPS, 4),
                                                 "avg_launch_ms": round(fwd_k, 4), "launches": fwd_n}}},
         "cpu_baseline": cpu,
         "pack_unpack": pack,
+        "server_tick": tick,
     }
     print(json.dumps(line), flush=True)
 
