@@ -15,6 +15,9 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libdistca_ca.so")
 SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]
+# The attention kernels exist once per element type: the same sources compiled again with -DDISTCA_F16 give the fp16
+# kernels and their launchers under names of their own; the entry points (compiled once) pick by distca_ca_params.dtype.
+F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-x", "hip",
@@ -66,9 +69,11 @@ def build_library(extra_flags: list[str] | None = None, verbose: bool = False, o
     lib_path = out_path or LIB_PATH
     obj_dir = os.path.join(PKG_DIR, "build", os.path.basename(lib_path))
     os.makedirs(obj_dir, exist_ok=True)
-    objs = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
-    with ThreadPoolExecutor(max_workers=min(len(SOURCES), 6)) as ex:
-        list(ex.map(lambda so: _compile(so[0], so[1], extra), zip(SOURCES, objs)))
+    jobs = [(s, os.path.join(obj_dir, os.path.splitext(s)[0] + ".o"), extra) for s in SOURCES]
+    jobs += [(s, os.path.join(obj_dir, os.path.splitext(s)[0] + "_f16.o"), extra + ["-DDISTCA_F16"]) for s in F16_SOURCES]
+    objs = [j[1] for j in jobs]
+    with ThreadPoolExecutor(max_workers=min(len(jobs), 8)) as ex:
+        list(ex.map(lambda j: _compile(*j), jobs))
     tmp = lib_path + ".tmp"
     cmd = [_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True)

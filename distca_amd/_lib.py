@@ -23,7 +23,7 @@ class CaParams(Structure):
         ("num_heads_q", c_int32), ("num_heads_kv", c_int32), ("head_dim", c_int32),
         ("max_seqlen_q", c_int32), ("max_seqlen_k", c_int32),
         ("softmax_scale", c_float), ("causal", c_int32), ("deterministic", c_int32),
-        ("reserved", c_int32),
+        ("dtype", c_int32),
     ]
 
 

@@ -45,6 +45,12 @@ int num_compute_units();
 // may both do the set-up, which is idempotent).
 bool device_setup_pending(int slot);
 void device_setup_done(int slot);
-enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotBwdLds64 = 2, kSlotCount = 3 };
+// Every kernel that needs such set-up exists once per element type; the fp16 builds of the sources use the upper half.
+enum { kSlotPerType = 3, kSlotCount = 2 * kSlotPerType };
+#ifdef DISTCA_F16
+enum { kSlotFwdLds = kSlotPerType + 0, kSlotBwdLds = kSlotPerType + 1, kSlotBwdLds64 = kSlotPerType + 2 };
+#else
+enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotBwdLds64 = 2 };
+#endif
 
 }  // namespace distca

@@ -3,12 +3,15 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/distca_ca.h"
+#include "common.h"
+
 namespace distca {
 
 struct BwdArgs {
-  const __bf16 *q, *k, *v, *dout;
+  const elem_t *q, *k, *v, *dout;
   const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and -delta
-  __bf16 *dq, *dk, *dv;
+  elem_t *dq, *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;
@@ -27,8 +30,33 @@ struct BwdArgs {
 };
 
 
+// The query side of a backward call: where dO, O, lse, q are read and dq is written.
+struct BwdQuerySide {
+  const void *dout, *q, *out;      // first byte of each part in token 0 of its region
+  const float *lse;                // [Hq][Tq], or nullptr with lse_tok
+  const void *lse_tok;             // first byte of the lse part in token 0, or nullptr
+  const int64_t *task_off;         // shared by dout, q, out, lse_tok; nullptr = packed tensors
+  int64_t tok_bytes;
+  void *dq;
+  const int64_t *dq_task_off;
+  int64_t dq_tok_bytes;
+};
+// The backward behind distca_ca_bwd and distca_ca_bwd_tokens, per element type (attn_bwd.hip compiled for each).
+int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+int run_bwd_f16(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+                const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+// The forward behind distca_ca_fwd_tokens, per element type (attn_fwd.hip compiled for each).
+int run_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v, void *out_base,
+                   const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q, const int32_t *cu_k,
+                   const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+int run_fwd_tokens_f16(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v, void *out_base,
+                       const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q, const int32_t *cu_k,
+                       const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+
 // The dK/dV kernel with 64 keys per wave (attn_bwd_dkdv64.hip): LDS bytes it needs, and its launch.
 int dkdv64_lds_bytes();
-int launch_dkdv64(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);
+int launch_dkdv64(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);       // bf16 elements
+int launch_dkdv64_f16(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);   // fp16 elements
 
 }  // namespace distca

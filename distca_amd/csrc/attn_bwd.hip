@@ -220,8 +220,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
       const int hg = (ok ? rho : 0) - tok * G;
       const int chunk = (lane & 15) ^ tile_swz(rl);
       const int64_t eo = qbase + (int64_t)tok * a.qs_tok_bytes + hg * (kHeadDim * 2);
-      const __bf16 *qs = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
-      const __bf16 *ds = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
+      const elem_t *qs = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
+      const elem_t *ds = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
       const uint32_t dst = lds0 + tile + wave * 4 * kTileRow;
       lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
       lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
   const int t_rd = (4 * g + i4) * kTileRow + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*(j&3) ^ 16*hi
 
-  bf16x8 kreg[8];  // this wave's 32 keys as B operand of S = Q K^T, all 8 steps over d
+  elemx8 kreg[8];  // this wave's 32 keys as B operand of S = Q K^T, all 8 steps over d
   f32x16 sacc, dpacc;
   // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
   auto phase_a = [&](int stage) {
@@ -257,12 +257,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
     // operands of step s+1 are requested before the MFMAs of step s are issued
     constexpr int kDa = 2;  // operand fetch distance in MFMA steps
-    bf16x8 qa[kDa], da[kDa], vb[kDa];
+    elemx8 qa[kDa], da[kDa], vb[kDa];
     auto load_a = [&](int s, int buf) {
       const int ao = a_rd ^ (s << 5);
-      qa[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + ao);
-      da[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + ao);
-      vb[buf] = *reinterpret_cast<const bf16x8 *>(lds + kVsOff + b_rd + 32 * s);
+      qa[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileQ + ao);
+      da[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileDO + ao);
+      vb[buf] = *reinterpret_cast<const elemx8 *>(lds + kVsOff + b_rd + 32 * s);
     };
 #pragma unroll
     for (int s = 0; s < kDa; ++s) load_a(s, s);
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
     }
   };
   // ---- phase B (VALU): P and dS, converted to bf16 B operands
-  bf16x8 pb[2], dsb[2];
+  elemx8 pb[2], dsb[2];
   auto phase_b = [&](int stage) {
     const uint8_t *stat = lds + kStatOff + stage * kStatBytes;
     const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   auto phase_c = [&](int stage) {
     const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
     constexpr int kDc = 2;  // operand fetch distance in MFMA steps
-    bf16x4 ct[kDc][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
+    elemx4 ct[kDc][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
     auto load_c = [&](int j, int buf) {
       const int lo = (16 * (j >> 2)) * kTileRow + (t_rd ^ ((j & 3) << 5));
       const int hi = (16 * (j >> 2) + 8) * kTileRow + (t_rd ^ ((j & 3) << 5) ^ 16);
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
   // query rows at the same time and find them in their XCD's L2.
   __syncthreads();
 #pragma unroll
-  for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const bf16x8 *>(lds + kKsOff + b_rd + 32 * s);
+  for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const elemx8 *>(lds + kKsOff + b_rd + 32 * s);
   __syncthreads();  // K has left LDS: its region now holds the tile ring
   if (niter > 0) {
     issue_tile(0, top - 1);
@@ -443,8 +443,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) 
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
           const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          *reinterpret_cast<bf16x4 *>(a.dk + off + d0) = cvt4(dkacc[db][4 * cq], dkacc[db][4 * cq + 1], dkacc[db][4 * cq + 2], dkacc[db][4 * cq + 3]);
-          *reinterpret_cast<bf16x4 *>(a.dv + off + d0) = cvt4(dvacc[db][4 * cq], dvacc[db][4 * cq + 1], dvacc[db][4 * cq + 2], dvacc[db][4 * cq + 3]);
+          *reinterpret_cast<elemx4 *>(a.dk + off + d0) = cvt4(dkacc[db][4 * cq], dkacc[db][4 * cq + 1], dkacc[db][4 * cq + 2], dkacc[db][4 * cq + 3]);
+          *reinterpret_cast<elemx4 *>(a.dv + off + d0) = cvt4(dvacc[db][4 * cq], dvacc[db][4 * cq + 1], dvacc[db][4 * cq + 2], dvacc[db][4 * cq + 3]);
         }
     }
   }
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   int row[MSUB], tok[MSUB], lim[MSUB];
   bool valid[MSUB];
   float lse2[MSUB], dsc[MSUB];
-  bf16x8 qf[MSUB][8], dof[MSUB][8];
+  elemx8 qf[MSUB][8], dof[MSUB][8];
 #pragma unroll
   for (int m = 0; m < MSUB; ++m) {
     row[m] = row_wg + (wave * MSUB + m) * 32 + l32;
@@ -513,11 +513,11 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       if (valid[m]) {
-        qf[m][s] = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s);
-        dof[m][s] = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
+        qf[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s);
+        dof[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
       } else {
-        qf[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        dof[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+        dof[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
       }
     }
   }
@@ -538,8 +538,8 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
   const int uwave = __builtin_amdgcn_readfirstlane(wave);
-  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
-  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
   constexpr int kRowsW = kDqKV / kWaves, kLdW = 2 * (kRowsW / 4);
   auto issue_kv = [&](int j, int stage, int i) {
     const bool is_k = i < kLdW / 2;
@@ -547,8 +547,8 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     const int r = kRowsW * uwave + 4 * ii + (lane >> 4);
     const int key = j * kDqKV + r;
     const int chunk = (lane & 15) ^ tile_swz(r);
-    const __bf16 *src = (is_k ? kbase : vbase) + (int64_t)key * kv_stride;
-    if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
+    const elem_t *src = (is_k ? kbase : vbase) + (int64_t)key * kv_stride;
+    if (key >= lk) src = reinterpret_cast<const elem_t *>(a.zero_row);
     const uint32_t dst = lds0 + stage * kDqStage + (is_k ? 0 : kDqTile) + (kRowsW * uwave + 4 * ii) * kDqRowB;
     lds_direct_load16_ptr(src + chunk * 8, dst);
   };
@@ -563,7 +563,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   auto issue_kv_whole = [&](int j, int stage, int i) {
     const bool is_k = i < kLdW / 2;
     const int ii = is_k ? i : i - kLdW / 2;
-    const __bf16 *tb = (is_k ? kbase : vbase) + (int64_t)j * kDqKV * kv_stride;
+    const elem_t *tb = (is_k ? kbase : vbase) + (int64_t)j * kDqKV * kv_stride;
     lds_direct_load16(tb, voff[ii], lds0 + stage * kDqStage + (is_k ? 0 : kDqTile) + (kRowsW * uwave + 4 * ii) * kDqRowB);
   };
 
@@ -625,12 +625,12 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       // operand fragments are requested kPf steps before the MFMAs that use them; the next tile's
       // loads go out one instruction per step
       constexpr int kPf = 1;
-      bf16x8 kf[kPf][2], vf[kPf][2];
+      elemx8 kf[kPf][2], vf[kPf][2];
       auto load_kv = [&](int s, int buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-          kf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kb * 32 * kDqRowB));
-          vf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kDqTile + kb * 32 * kDqRowB));
+          kf[buf][kb] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kb * 32 * kDqRowB));
+          vf[buf][kb] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(k_ad[s] + stage * kDqStage + kDqTile + kb * 32 * kDqRowB));
         }
       };
 #pragma unroll
@@ -651,7 +651,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       }
       // ---- P, dS (one query row per lane) and the bf16 B operand of the dQ product
       const bool need_mask = key0 + kDqKV - 1 > lim_first;
-      bf16x8 dsf[MSUB][4];
+      elemx8 dsf[MSUB][4];
 #pragma unroll
       for (int m = 0; m < MSUB; ++m) {
         // the masked form only for tiles that straddle the diagonal or the end of the prefix (uniform branch)
@@ -678,7 +678,7 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
       }
       // ---- dQ^T += K^T dS^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
       constexpr int kPfT = 4;
-      bf16x4 ktf[kPfT][2];
+      elemx4 ktf[kPfT][2];
       auto load_t = [&](int u, int buf) {  // u = 4*t + db
         const uint32_t ko = stage * kDqStage + 16 * (u >> 2) * kDqRowB;
         ktf[buf][0] = lds_read_tr(lds_ptr(t_ad[u & 3] + ko));
@@ -708,13 +708,13 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   for (int m = 0; m < MSUB; ++m) {
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
-      __bf16 *op = reinterpret_cast<__bf16 *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
+      elem_t *op = reinterpret_cast<elem_t *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
           const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          *reinterpret_cast<bf16x4 *>(op + d0) =
+          *reinterpret_cast<elemx4 *>(op + d0) =
               cvt4(dqacc[m][db][4 * cq], dqacc[m][db][4 * cq + 1], dqacc[m][db][4 * cq + 2], dqacc[m][db][4 * cq + 3]);
         }
     }
@@ -757,8 +757,8 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restr
       tok_start = t * tok_bytes;
     }
     const int64_t eo = tok_start + (int64_t)h * (kHeadDim * 2) + sub * 16;
-    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(dout + eo);
-    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(out + eo);
+    const elemx8 a = *reinterpret_cast<const elemx8 *>(dout + eo);
+    const elemx8 b = *reinterpret_cast<const elemx8 *>(out + eo);
 #pragma unroll
     for (int i = 0; i < 8; ++i) s += (float)a[i] * (float)b[i];
   }
@@ -805,13 +805,13 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(u32x4 *__restrict__ p, i
 }
 
 // fp32 accumulator -> bf16, 8 elements per thread
-__global__ __launch_bounds__(256) void cvt_bf16_kernel(const float *__restrict__ src, __bf16 *__restrict__ dst, int64_t n8) {
+__global__ __launch_bounds__(256) void cvt_elem_kernel(const float *__restrict__ src, elem_t *__restrict__ dst, int64_t n8) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (; i < n8; i += stride) {
     const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + 2 * i);
     const f32x4 y = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + 2 * i + 1);
-    reinterpret_cast<bf16x8 *>(dst)[i] = cvt8(x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]);
+    reinterpret_cast<elemx8 *>(dst)[i] = cvt8(x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]);
   }
 }
 
@@ -843,6 +843,7 @@ int grid_for(int64_t work_items) {
 
 using namespace distca;
 
+#ifndef DISTCA_F16
 extern "C" int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p) {
   if (!p) return fail(DISTCA_E_INVALID, "bwd_workspace_bytes: null params");
   int rc = validate_params(p);
@@ -851,29 +852,13 @@ extern "C" int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p) {
   return bwd_layout(p, true).total;
 }
 
-namespace {
-// The query side of a backward call: where dO, O, lse, q are read and dq is written.
-struct BwdQuerySide {
-  const void *dout, *q, *out;      // first byte of each part in token 0 of its region
-  const float *lse;                // [Hq][Tq], or nullptr with lse_tok
-  const void *lse_tok;             // first byte of the lse part in token 0, or nullptr
-  const int64_t *task_off;         // shared by dout, q, out, lse_tok; nullptr = packed tensors
-  int64_t tok_bytes;
-  void *dq;
-  const int64_t *dq_task_off;
-  int64_t dq_tok_bytes;
-};
-int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
-            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
-}  // namespace
-
 extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
                              void *dq, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
                              const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
   const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2;
   const BwdQuerySide qs{dout, q, out, lse, nullptr, nullptr, row_bytes, dq, nullptr, row_bytes};
-  return run_bwd(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
 }
 
 extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off, int64_t req_tok_bytes, const void *k,
@@ -896,12 +881,13 @@ extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_tas
   // [dO | O | lse | q | pad]
   const BwdQuerySide qs{r, r ? r + 2 * row_bytes + lse_bytes : nullptr, r ? r + row_bytes : nullptr, nullptr,
                         r ? r + 2 * row_bytes : nullptr, req_task_off, req_tok_bytes, dq_base, dq_task_off, dq_tok_bytes};
-  return run_bwd(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
 }
+#endif  // !DISTCA_F16
 
-namespace {
-int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
-            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+namespace distca {
+int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+                       const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
   const void *dout = qs.dout, *q = qs.q, *out = qs.out;
   void *dq = qs.dq;
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
@@ -950,9 +936,9 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
                      (float *)(ws + w.delta), (float *)(ws + w.lse2), rows, p->num_heads_q, p->total_q, p->softmax_scale);
 
   BwdArgs a;
-  a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v; a.dout = (const __bf16 *)dout;
+  a.q = (const elem_t *)q; a.k = (const elem_t *)k; a.v = (const elem_t *)v; a.dout = (const elem_t *)dout;
   a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta);
-  a.dq = (__bf16 *)dq; a.dk = (__bf16 *)dk; a.dv = (__bf16 *)dv;
+  a.dq = (elem_t *)dq; a.dk = (elem_t *)dk; a.dv = (elem_t *)dv;
   a.qs_task_off = qs.task_off; a.qs_tok_bytes = qs.tok_bytes; a.dq_task_off = qs.dq_task_off; a.dq_tok_bytes = qs.dq_tok_bytes;
   a.dk_acc = use_acc ? (float *)(ws + w.dk_acc) : nullptr;
   a.dv_acc = use_acc ? (float *)(ws + w.dv_acc) : nullptr;
@@ -988,7 +974,7 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
 #if DISTCA_DKDV64
-    rc = launch_dkdv64(a, grid, use_acc, s);
+    rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, s);
     if (rc) return rc;
 #else
     if (use_acc)
@@ -1012,10 +998,10 @@ int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void
     hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
   }
   if (use_acc) {
-    hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (__bf16 *)dk, kv_elems / 8);
-    hipLaunchKernelGGL(cvt_bf16_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dv_acc), (__bf16 *)dv, kv_elems / 8);
+    hipLaunchKernelGGL(cvt_elem_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (elem_t *)dk, kv_elems / 8);
+    hipLaunchKernelGGL(cvt_elem_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dv_acc), (elem_t *)dv, kv_elems / 8);
   }
   (void)q_elems;
   return check_launch("ca_bwd");
 }
-}  // namespace
+}  // namespace distca

@@ -64,11 +64,11 @@ __device__ __forceinline__ void fence() { __builtin_amdgcn_sched_barrier(0); }
 // so does not space its result from the vector instructions that read it (11 quad-cycles for this MFMA): the
 // order of a block's instructions below keeps at least one later MFMA, which cannot start before the pipe has
 // finished with the one in question, between every such MFMA and the first read of its result.
-__device__ __forceinline__ void mfma32_v(f32x16 &acc, bf16x8 a, bf16x8 b) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+__device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
-__device__ __forceinline__ void mfma32_v0(f32x16 &acc, bf16x8 a, bf16x8 b) {  // acc = A B
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+__device__ __forceinline__ void mfma32_v0(f32x16 &acc, elemx8 a, elemx8 b) {  // acc = A B
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
 }
 
 template <bool ALIAS>
@@ -120,20 +120,20 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
 
   // ---- K of the wave's keys as B operands (lane holds key 32 kb + l32, d = 16 s + 8 g .. +7); V of the same keys
   // into LDS, read back by this wave only
-  bf16x8 kreg[2][8];
+  elemx8 kreg[2][8];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int key = kw0 + 32 * kb + l32;
     const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim + 8 * g;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      bf16x8 kf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0}, vf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      elemx8 kf = elemx8{0, 0, 0, 0, 0, 0, 0, 0}, vf = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
       if (key < lk) {
-        kf = *reinterpret_cast<const bf16x8 *>(a.k + off + 16 * s);
-        vf = *reinterpret_cast<const bf16x8 *>(a.v + off + 16 * s);
+        kf = *reinterpret_cast<const elemx8 *>(a.k + off + 16 * s);
+        vf = *reinterpret_cast<const elemx8 *>(a.v + off + 16 * s);
       }
       kreg[kb][s] = kf;
-      *reinterpret_cast<bf16x8 *>(lds + kVOff + (wave * 64 + 32 * kb + l32) * kVPitch + 32 * s + 16 * g) = vf;
+      *reinterpret_cast<elemx8 *>(lds + kVOff + (wave * 64 + 32 * kb + l32) * kVPitch + 32 * s + 16 * g) = vf;
     }
   }
   const int v_rd = kVOff + (wave * 64 + l32) * kVPitch + 16 * g;  // + 32*kb*kVPitch + 32*s
@@ -222,8 +222,8 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       const int hg = (ok ? rho : 0) - tok * G;
       const int chunk = (lane & 15) ^ tile_swz(rl);
       const int64_t eo = qbase + (int64_t)tok * a.qs_tok_bytes + hg * (kHeadDim * 2);
-      const __bf16 *qs = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
-      const __bf16 *ds = reinterpret_cast<const __bf16 *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
+      const elem_t *qs = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
+      const elem_t *ds = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
       const uint32_t dst = lds0 + tile + (wave * 8 + 4 * i) * kRow;
       lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
       lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
@@ -269,12 +269,12 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       }
     }
     // ---- step 1: S = Q K^T
-    bf16x8 qa[2], da[2], vb[2][2];
-    auto load_q = [&](int s, int buf) { qa[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileQ + (a_rd ^ (s << 5))); };
+    elemx8 qa[2], da[2], vb[2][2];
+    auto load_q = [&](int s, int buf) { qa[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileQ + (a_rd ^ (s << 5))); };
     auto load_dv = [&](int s, int buf) {
-      da[buf] = *reinterpret_cast<const bf16x8 *>(tile + kTileDO + (a_rd ^ (s << 5)));
-      vb[buf][0] = *reinterpret_cast<const bf16x8 *>(lds + v_rd + 32 * s);
-      vb[buf][1] = *reinterpret_cast<const bf16x8 *>(lds + v_rd + 32 * kVPitch + 32 * s);
+      da[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileDO + (a_rd ^ (s << 5)));
+      vb[buf][0] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * s);
+      vb[buf][1] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * kVPitch + 32 * s);
     };
     load_q(0, 0);
     load_q(1, 1);
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     }
 
     // ---- step 2: dP = dO V^T; beside the MFMAs, P = exp2(S c - lse2) of two elements per MFMA
-    bf16x8 pb[2][2], dsb[2][2];
+    elemx8 pb[2][2], dsb[2][2];
     auto p_elem = [&](int kb, int r) {
       float p = fast_exp2(__builtin_fmaf(sacc[kb][r], c, -lse_buf[(r >> 2) & 1][r & 3]));
       if constexpr (kMasked) {
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       pb[kb][t] = cvt8(sacc[kb][r0], sacc[kb][r0 + 1], sacc[kb][r0 + 2], sacc[kb][r0 + 3], sacc[kb][r0 + 4], sacc[kb][r0 + 5],
                        sacc[kb][r0 + 6], sacc[kb][r0 + 7]);
     };
-    bf16x4 ct[2][2];  // transposed fragments [buffer][lo, hi]
+    elemx4 ct[2][2];  // transposed fragments [buffer][lo, hi]
     auto load_t = [&](int which, int j, int buf) {
       const int lo = (16 * (j >> 2)) * kRow + (t_rd ^ ((j & 3) << 5));
       const int hi = (16 * (j >> 2) + 8) * kRow + (t_rd ^ ((j & 3) << 5) ^ 16);
@@ -346,7 +346,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     };
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const bf16x8 dot = cat4(ct[j & 1][0], ct[j & 1][1]);
+      const elemx8 dot = cat4(ct[j & 1][0], ct[j & 1][1]);
       fence();
       dvacc[0][j & 3] = mfma32(dot, pb[0][j >> 2], dvacc[0][j & 3]);
       fence();
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     // ---- step 4: dK^T += Q^T dS
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const bf16x8 qt = cat4(ct[j & 1][0], ct[j & 1][1]);
+      const elemx8 qt = cat4(ct[j & 1][0], ct[j & 1][1]);
       fence();
       dkacc[0][j & 3] = mfma32(qt, dsb[0][j >> 2], dkacc[0][j & 3]);
       dkacc[1][j & 3] = mfma32(qt, dsb[1][j >> 2], dkacc[1][j & 3]);
@@ -474,9 +474,9 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
 #pragma unroll
           for (int cq = 0; cq < 4; ++cq) {
             const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-            *reinterpret_cast<bf16x4 *>(a.dk + off + d0) =
+            *reinterpret_cast<elemx4 *>(a.dk + off + d0) =
                 cvt4(dkacc[kb][db][4 * cq], dkacc[kb][db][4 * cq + 1], dkacc[kb][db][4 * cq + 2], dkacc[kb][db][4 * cq + 3]);
-            *reinterpret_cast<bf16x4 *>(a.dv + off + d0) =
+            *reinterpret_cast<elemx4 *>(a.dv + off + d0) =
                 cvt4(dvacc[kb][db][4 * cq], dvacc[kb][db][4 * cq + 1], dvacc[kb][db][4 * cq + 2], dvacc[kb][db][4 * cq + 3]);
           }
       }
@@ -486,9 +486,11 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
 
 }  // namespace
 
+#ifndef DISTCA_F16
 int dkdv64_lds_bytes() { return kLds; }
+#endif
 
-int launch_dkdv64(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream) {
+int DISTCA_FN(launch_dkdv64)(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream) {
   if (device_setup_pending(kSlotBwdLds64)) {
     hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);

@@ -34,7 +34,9 @@ constexpr int kBwdRows = 32;
 constexpr int kBwdKV = 256;
 
 inline int validate_params(const distca_ca_params *p) {
-  if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: this build has kernels for head_dim 128 only", p->head_dim);
+  if (p->head_dim != kHeadDim) return fail(DISTCA_E_UNSUPPORTED, "head_dim=%d: the kernels are built for head_dim 128 (smaller ones can be zero-padded to it)", p->head_dim);
+  if (p->dtype != 0 && p->dtype != DISTCA_DTYPE_BF16 && p->dtype != DISTCA_DTYPE_F16)
+    return fail(DISTCA_E_UNSUPPORTED, "dtype=%d: the attention kernels take bf16 (%d, or 0) or fp16 (%d) elements", p->dtype, DISTCA_DTYPE_BF16, DISTCA_DTYPE_F16);
   if (p->num_heads_q <= 0 || p->num_heads_kv <= 0 || p->num_heads_q % p->num_heads_kv)
     return fail(DISTCA_E_INVALID, "num_heads_q=%d must be a positive multiple of num_heads_kv=%d", p->num_heads_q, p->num_heads_kv);
   if (p->num_heads_kv > kSchedMaxHeads) return fail(DISTCA_E_UNSUPPORTED, "num_heads_kv=%d: at most %d kv heads", p->num_heads_kv, kSchedMaxHeads);

@@ -26,6 +26,7 @@
 #include <mutex>
 
 #include "api_util.h"
+#include "attn_bwd.h"
 #include "attn_cfg.h"
 #include "common.h"
 
@@ -41,8 +42,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 struct FwdArgs {
-  const __bf16 *q, *k, *v;
-  __bf16 *out;
+  const elem_t *q, *k, *v;
+  elem_t *out;
   float *lse;
   const int32_t *cu_q, *cu_k, *kv_off;
   const int32_t *sched;  // schedule workspace
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   uint8_t *obytes = reinterpret_cast<uint8_t *>(a.out) + (a.out_task_off ? a.out_task_off[task] : (int64_t)q0 * a.out_tok_bytes);
   int row[MSUB], tok[MSUB], lim[MSUB];
   bool valid[MSUB];
-  const __bf16 *qptr[MSUB];
+  const elem_t *qptr[MSUB];
 #pragma unroll
   for (int m = 0; m < MSUB; ++m) {
     row[m] = row_wg + (wave * MSUB + m) * 32 + l32;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     int lm = a.causal ? tok[m] + shift : lk - 1;
     if (lm > lk - 1) lm = lk - 1;
     lim[m] = lm;
-    qptr[m] = reinterpret_cast<const __bf16 *>(qbytes + (int64_t)tok[m] * a.q_tok_bytes) + (kvh * G + hg) * kHeadDim;
+    qptr[m] = reinterpret_cast<const elem_t *>(qbytes + (int64_t)tok[m] * a.q_tok_bytes) + (kvh * G + hg) * kHeadDim;
   }
   // wave-uniform limits: first row's limit decides whether a tile needs masking, last row's
   // whether the wave has anything to do in it.
@@ -120,13 +121,13 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   }
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds row l32, d = 16*s + 8*g .. +7
-  bf16x8 qf[MSUB][8];
+  elemx8 qf[MSUB][8];
 #pragma unroll
   for (int m = 0; m < MSUB; ++m) {
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      if (valid[m]) qf[m][s] = *reinterpret_cast<const bf16x8 *>(qptr[m] + 16 * s + 8 * g);
-      else qf[m][s] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (valid[m]) qf[m][s] = *reinterpret_cast<const elemx8 *>(qptr[m] + 16 * s + 8 * g);
+      else qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
 
@@ -135,18 +136,18 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
   const int uwave = __builtin_amdgcn_readfirstlane(wave);
-  const __bf16 *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
-  const __bf16 *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
   // a wave brings kRowsW rows of a K tile or of a V tile, four rows per instruction
   constexpr int kRowsW = kFwdKV / kFwdWaves, kLdW = kRowsW / 4;
-  auto issue_rows = [&](const __bf16 *base, int j, uint32_t tile_off) {
+  auto issue_rows = [&](const elem_t *base, int j, uint32_t tile_off) {
 #pragma unroll
     for (int i = 0; i < kLdW; ++i) {
       const int r = kRowsW * uwave + 4 * i + (lane >> 4);
       const int key = j * kFwdKV + r;
       const int chunk = (lane & 15) ^ tile_swz(r);
-      const __bf16 *src = base + (int64_t)key * kv_stride;
-      if (key >= lk) src = reinterpret_cast<const __bf16 *>(a.zero_row);
+      const elem_t *src = base + (int64_t)key * kv_stride;
+      if (key >= lk) src = reinterpret_cast<const elem_t *>(a.zero_row);
       lds_direct_load16_ptr(src + chunk * 8, lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
     }
   };
@@ -158,8 +159,8 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     const int r = kRowsW * uwave + 4 * i + (lane >> 4);
     voff[i] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
   }
-  auto issue_rows_fast = [&](const __bf16 *base, int j, uint32_t tile_off) {
-    const __bf16 *tb = base + (int64_t)j * kFwdKV * kv_stride;
+  auto issue_rows_fast = [&](const elem_t *base, int j, uint32_t tile_off) {
+    const elem_t *tb = base + (int64_t)j * kFwdKV * kv_stride;
 #pragma unroll
     for (int i = 0; i < kLdW; ++i) lds_direct_load16(tb, voff[i], lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
   };
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     asm volatile("" : "+v"(k_ad[i]), "+v"(v_ad[i]));
   }
   f32x16 sacc[MSUB][2];
-  bf16x8 pf[MSUB][4];
+  elemx8 pf[MSUB][4];
   auto tile_active = [&](int j) { return wave_live && j * kFwdKV <= lim_last; };
 
   // ---- S^T = K Q^T : [64 keys] x [32*MSUB rows]
@@ -217,10 +218,10 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[m][kb][r] = 0.f;
     constexpr int kPf = 2;  // K fragments are requested kPf steps before the MFMAs that use them
-    bf16x8 kf[kPf][2];
+    elemx8 kf[kPf][2];
     auto load_k = [&](int s, int buf) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *static_cast<const DISTCA_LDS bf16x8 *>(lds_ptr(k_ad[s] + decltype(par)::value * kKTile + kb * 32 * kRowB));
+      for (int kb = 0; kb < 2; ++kb) kf[buf][kb] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(k_ad[s] + decltype(par)::value * kKTile + kb * 32 * kRowB));
     };
 #pragma unroll
     for (int s = 0; s < kPf; ++s) load_k(s, s);
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   // ---- O^T += V^T P^T : [128 d] x [32*MSUB rows], contraction over the 64 keys
   auto phase_pv = [&](int j, auto par) __attribute__((always_inline)) {
     constexpr int kPfV = 4;  // V^T fragments are requested four MFMAs ahead
-    bf16x4 vf[kPfV][2];
+    elemx4 vf[kPfV][2];
     auto load_v = [&](int u, int buf) {  // u = 4*t + db
       const uint32_t vo = decltype(par)::value * kVTile + 16 * (u >> 2) * kRowB;
       vf[buf][0] = lds_read_tr(lds_ptr(v_ad[u & 3] + vo));
@@ -387,16 +388,16 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
       uint8_t *otok = obytes + (int64_t)tok[m] * a.out_tok_bytes;
-      __bf16 *op = reinterpret_cast<__bf16 *>(otok) + (kvh * G + hg) * kHeadDim;
+      elem_t *op = reinterpret_cast<elem_t *>(otok) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
           // registers 4*cq .. 4*cq+3 of block db hold d0 .. d0+3
           const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          const bf16x4 o4 = cvt4(oacc[m][db][4 * cq] * inv, oacc[m][db][4 * cq + 1] * inv, oacc[m][db][4 * cq + 2] * inv,
+          const elemx4 o4 = cvt4(oacc[m][db][4 * cq] * inv, oacc[m][db][4 * cq + 1] * inv, oacc[m][db][4 * cq + 2] * inv,
                                  oacc[m][db][4 * cq + 3] * inv);
-          *reinterpret_cast<bf16x4 *>(op + d0) = o4;
+          *reinterpret_cast<elemx4 *>(op + d0) = o4;
         }
       if (g == 0) {
         const float lse = l_tot > 0.f ? (m_run[m] * c + fast_log2(l_tot)) * kLn2 : -INFINITY;
@@ -420,6 +421,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
 
 using namespace distca;
 
+#ifndef DISTCA_F16
 // Scratch memory of distca_ca_fwd_noalloc: the forward's work list, zero row and ticket counters, which every other
 // entry point takes from the caller's workspace.  One copy per GPU, held until the process ends.  The name below is
 // a host-side stand-in, never a device address: host code uses the per-device address from hipGetSymbolAddress.
@@ -459,7 +461,12 @@ extern "C" int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p) {
 extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,
                                     const void *v, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes,
                                     float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
-                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_fwd_tokens_f16 : run_fwd_tokens)(q_base, q_task_off, q_tok_bytes, k, v, out_base, out_task_off,
+                                                                              out_tok_bytes, lse, cu_q, cu_k, kv_off, p, workspace,
+                                                                              workspace_bytes, stream);
+}
 
 extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
@@ -488,10 +495,13 @@ extern "C" int distca_ca_fwd_noalloc(const void *q, const void *k, const void *v
   return distca_ca_fwd(q, k, v, out, lse, cu_q, cu_k, kv_off, p, ws, kNoAllocScratchBytes, stream);
 }
 
-extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,
-                                    const void *v, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes,
-                                    float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
-                                    const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+#endif  // !DISTCA_F16
+
+namespace distca {
+int DISTCA_FN(run_fwd_tokens)(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v,
+                              void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q,
+                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
+                              int64_t workspace_bytes, void *stream) {
   const void *q = q_base;
   void *out = out_base;
   if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
@@ -517,8 +527,8 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   if (rc) return rc;
 
   FwdArgs a;
-  a.q = (const __bf16 *)q; a.k = (const __bf16 *)k; a.v = (const __bf16 *)v;
-  a.out = (__bf16 *)out; a.lse = lse;
+  a.q = (const elem_t *)q; a.k = (const elem_t *)k; a.v = (const elem_t *)v;
+  a.out = (elem_t *)out; a.lse = lse;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
   a.sched = (const int32_t *)workspace;
   a.zero_row = (const uint8_t *)workspace + sched_zero_row_off(p->num_tasks, max_items);
@@ -541,3 +551,4 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
   }
   return check_launch("ca_fwd");
 }
+}  // namespace distca

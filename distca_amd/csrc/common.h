@@ -5,9 +5,20 @@
 
 namespace distca {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// The 16-bit element type of q, k, v, out and the gradients.  The attention sources are compiled twice: as they are
+// for bf16, and with -DDISTCA_F16 for IEEE half precision; DISTCA_FN gives what they export a name per element type.
+#ifdef DISTCA_F16
+typedef _Float16 elem_t;
+#define DISTCA_FN(name) name##_f16
+#define DISTCA_MFMA32_ASM "v_mfma_f32_32x32x16_f16"
+#else
+typedef __bf16 elem_t;
+#define DISTCA_FN(name) name
+#define DISTCA_MFMA32_ASM "v_mfma_f32_32x32x16_bf16"
+#endif
+typedef elem_t elemx8 __attribute__((ext_vector_type(8)));
+typedef elem_t elemx4 __attribute__((ext_vector_type(4)));
+typedef elem_t elemx2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -23,8 +34,12 @@ typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 //   A operand: lane l holds row l%32, k = 8*(l/32) .. +7
 //   B operand: lane l holds col l%32, k = 8*(l/32) .. +7
 //   C/D:       lane l holds col l%32, register r holds row 8*(r/4) + 4*(l/32) + r%4
-__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+__device__ __forceinline__ f32x16 mfma32(elemx8 a, elemx8 b, f32x16 c) {
+#ifdef DISTCA_F16
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#else
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 // Row index (0..31) inside a 32x32 accumulator block for register r of lane-half g.
@@ -37,22 +52,22 @@ __device__ __forceinline__ constexpr int acc_row(int r, int g) { return 8 * (r >
 // column c0 + L of rows r0 .. r0+3.
 // An LDS pointer from a 32-bit LDS address.
 __device__ __forceinline__ const DISTCA_LDS void *lds_ptr(uint32_t addr) { return reinterpret_cast<const DISTCA_LDS void *>(static_cast<uintptr_t>(addr)); }
-__device__ __forceinline__ bf16x4 lds_read_tr(const DISTCA_LDS void *p) {
+__device__ __forceinline__ elemx4 lds_read_tr(const DISTCA_LDS void *p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DISTCA_LDS s16x4 *)p);
-  return __builtin_bit_cast(bf16x4, v);
+  return __builtin_bit_cast(elemx4, v);
 }
 
-__device__ __forceinline__ bf16x8 cat4(bf16x4 lo, bf16x4 hi) {
+__device__ __forceinline__ elemx8 cat4(elemx4 lo, elemx4 hi) {
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-__device__ __forceinline__ bf16x8 cvt8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
+__device__ __forceinline__ elemx8 cvt8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
   f32x8 v = {a0, a1, a2, a3, a4, a5, a6, a7};
-  return __builtin_convertvector(v, bf16x8);
+  return __builtin_convertvector(v, elemx8);
 }
-__device__ __forceinline__ bf16x4 cvt4(float a0, float a1, float a2, float a3) {
+__device__ __forceinline__ elemx4 cvt4(float a0, float a1, float a2, float a3) {
   f32x4 v = {a0, a1, a2, a3};
-  return __builtin_convertvector(v, bf16x4);
+  return __builtin_convertvector(v, elemx4);
 }
 
 // max / sum of x over the lane pair (l, l^32).

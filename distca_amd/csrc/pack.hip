@@ -253,6 +253,7 @@ template <>
 struct Add<__bf16> {
   // bf16 + bf16: exact in fp32 up to one rounding that never lands on a bf16 tie, so
   // fp32 add followed by round-to-nearest-even equals the correctly rounded bf16 sum.
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
   static __device__ __forceinline__ u32x4 apply(u32x4 a, u32x4 b) {
     bf16x8 x = __builtin_bit_cast(bf16x8, a), y = __builtin_bit_cast(bf16x8, b);
     f32x8 fx = __builtin_convertvector(x, f32x8), fy = __builtin_convertvector(y, f32x8);

@@ -60,9 +60,27 @@ class FlashAttnArgs:
             self.deterministic = os.getenv("NVTE_ALLOW_NONDETERMINISTIC_ALGO", "0") != "1"
 
 
-def _params(num_tasks, total_q, total_k, hq, hkv, d, max_q, max_k, scale, causal, deterministic) -> _lib.CaParams:
+# element types of the attention kernels -> DISTCA_DTYPE_* of include/distca_ca.h
+_ELEM_CODE = {torch.float16: 1, torch.bfloat16: 2}
+HEAD_DIM = 128   # what the kernels are built for; smaller head dimensions are zero-padded to it on the way in
+
+
+def _params(num_tasks, total_q, total_k, hq, hkv, d, max_q, max_k, scale, causal, deterministic,
+            dtype: torch.dtype = torch.bfloat16) -> _lib.CaParams:
     return _lib.CaParams(num_tasks, total_q, total_k, hq, hkv, d, int(max_q), int(max_k), float(scale),
-                         1 if causal else 0, 1 if deterministic else 0, 0)
+                         1 if causal else 0, 1 if deterministic else 0, _ELEM_CODE[dtype])
+
+
+def _pad_head_dim(t: Tensor) -> Tensor:
+    """[T, H, d] -> [T, H, 128] with zeros behind the d values of every head (the reference pads to a multiple of 8,
+    fused_comm_attn.py:125-129, and leaves the rest to flash-attn; here the kernels have one head dimension).
+    Zero dimensions add nothing to q.k, and the output's and the gradients' padded dimensions come back as zeros."""
+    d = t.shape[-1]
+    if d == HEAD_DIM:
+        return t
+    if d > HEAD_DIM or d % 8:
+        raise RuntimeError(f"head_dim={d}: must be a multiple of 8 and at most {HEAD_DIM}")
+    return torch.nn.functional.pad(t, (0, HEAD_DIM - d))
 
 
 def _check_qkv(q: Tensor, k: Tensor, v: Tensor, cu_q: Tensor, cu_k: Tensor, kv_off: Optional[Tensor]):
@@ -71,8 +89,8 @@ def _check_qkv(q: Tensor, k: Tensor, v: Tensor, cu_q: Tensor, cu_k: Tensor, kv_o
             raise RuntimeError(f"{name} must have shape [tokens, heads, head_dim]")
         if not t.is_cuda:
             raise RuntimeError(f"{name} must be on CUDA")
-        if t.dtype != torch.bfloat16:
-            raise RuntimeError(f"{name} must be bfloat16 (got {t.dtype})")
+        if t.dtype not in _ELEM_CODE or t.dtype != q.dtype:
+            raise RuntimeError(f"{name} must be bfloat16 or float16, the same for q, k and v (got {t.dtype})")
         if not t.is_contiguous():
             raise RuntimeError(f"{name} must be contiguous")
     if k.shape != v.shape:
@@ -100,15 +118,20 @@ def _workspace(given: Optional[Tensor], need: int, device) -> Tensor:
 def ca_varlen_fwd(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor, cu_seqlens_k: Tensor,
                   max_seqlen_q: int, max_seqlen_k: int, softmax_scale: Optional[float] = None, causal: bool = True,
                   kv_task_offsets: Optional[Tensor] = None, workspace: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
-    """q [Tq,Hq,D], k,v [Tk,Hkv,D] bf16 -> (out [Tq,Hq,D] bf16, softmax_lse [Hq,Tq] fp32).
+    """q [Tq,Hq,D], k,v [Tk,Hkv,D] bf16 or fp16 -> (out [Tq,Hq,D] in the same type, softmax_lse [Hq,Tq] fp32).
     `workspace` (uint8 CUDA tensor of at least distca_ca_fwd_workspace_bytes) is allocated
-    per call when omitted."""
+    per call when omitted.  A head dimension below 128 (multiple of 8) goes through zero-padded copies."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
+    scale = softmax_scale if softmax_scale is not None else q.shape[2] ** (-0.5)
+    if q.shape[2] != HEAD_DIM:
+        d = q.shape[2]
+        out, lse = ca_varlen_fwd(_pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v), cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
+                                 max_seqlen_k, scale, causal, kv_task_offsets, workspace)
+        return out[..., :d].contiguous(), lse
     tq, hq, d = q.shape
     tk, hkv, _ = k.shape
-    scale = softmax_scale if softmax_scale is not None else d ** (-0.5)
     lib = _lib.load()
-    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, False)
+    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, False, q.dtype)
     need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
     if need < 0:
         _lib.check(int(need), "ca_varlen_fwd")
@@ -130,14 +153,24 @@ def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, so
                   kv_task_offsets: Optional[Tensor] = None,
                   dq: Optional[Tensor] = None, dk: Optional[Tensor] = None, dv: Optional[Tensor] = None,
                   workspace: Optional[Tensor] = None):
-    """Gradients (dq, dk, dv) in bf16; written into dq/dk/dv when given (the reference's
+    """Gradients (dq, dk, dv) in the type of q; written into dq/dk/dv when given (the reference's
     flash-attn backward fills caller-allocated tensors, fused_comm_attn.py:236,259-272)."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k, kv_task_offsets)
     tq, hq, d = q.shape
     tk, hkv, _ = k.shape
     for name, t in (("dout", dout), ("out", out)):
-        if t.shape != q.shape or t.dtype != torch.bfloat16 or not t.is_cuda:
-            raise RuntimeError(f"{name} must be a bfloat16 CUDA tensor shaped like q")
+        if t.shape != q.shape or t.dtype != q.dtype or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a CUDA tensor with the shape and type of q")
+    if d != HEAD_DIM:
+        scale = softmax_scale if softmax_scale is not None else d ** (-0.5)
+        grads = ca_varlen_bwd(_pad_head_dim(dout), _pad_head_dim(q), _pad_head_dim(k), _pad_head_dim(v), _pad_head_dim(out),
+                              softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, scale, causal, deterministic,
+                              kv_task_offsets, workspace=workspace)
+        res = []
+        for g, given in zip(grads, (dq, dk, dv)):
+            g = g[..., :d]
+            res.append(g.contiguous() if given is None else given.copy_(g))
+        return tuple(res)
     dout = dout.contiguous()
     out = out.contiguous()
     if softmax_lse.shape != (hq, tq) or softmax_lse.dtype != torch.float32:
@@ -145,7 +178,7 @@ def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, so
     softmax_lse = softmax_lse.contiguous()
     scale = softmax_scale if softmax_scale is not None else d ** (-0.5)
     lib = _lib.load()
-    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, deterministic)
+    p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_k, scale, causal, deterministic, q.dtype)
     need = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
     if need < 0:
         _lib.check(int(need), "ca_varlen_bwd")
@@ -153,8 +186,8 @@ def ca_varlen_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, so
     dk = torch.empty_like(k) if dk is None else dk
     dv = torch.empty_like(v) if dv is None else dv
     for name, t, ref in (("dq", dq, q), ("dk", dk, k), ("dv", dv, v)):
-        if t.shape != ref.shape or t.dtype != torch.bfloat16 or not t.is_contiguous() or not t.is_cuda:
-            raise RuntimeError(f"{name} must be a contiguous bfloat16 CUDA tensor shaped like its input")
+        if t.shape != ref.shape or t.dtype != q.dtype or not t.is_contiguous() or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a contiguous CUDA tensor with the shape and type of its input")
     ws = _workspace(workspace, int(need), q.device)
     with torch.cuda.device(q.device):
         rc = lib.distca_ca_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
@@ -292,11 +325,12 @@ def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdM
     send buffer."""
     dev = recv_buffer.device
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
-    shared = meta.shared_kv if in_place and dtype == torch.bfloat16 else None
+    in_place = in_place and dtype in _ELEM_CODE and d == HEAD_DIM
+    shared = meta.shared_kv if in_place else None
     k_rows = shared.num_rows if shared is not None else meta.recv_k_shape[0]
     recv_k = torch.empty((k_rows, meta.recv_k_shape[1]), dtype=dtype, device=dev)
     recv_v = torch.empty_like(recv_k)
-    if in_place and dtype == torch.bfloat16:
+    if in_place:
         kv_off = getattr(fa_params, "kv_task_offsets", None)
         if shared is not None:
             # one copy of every K/V shard, documents contiguous: every task reads its prefix in place
@@ -312,7 +346,7 @@ def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdM
         cu_q, cu_k = fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv
         assert fa_args.causal and fa_args.window_size == (-1, -1) and fa_args.dropout_p == 0.0
         p = _params(cu_q.shape[0] - 1, tq, tk, hq, hkv, d, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, scale,
-                    fa_args.causal, False)
+                    fa_args.causal, False, dtype)
         need = lib.distca_ca_fwd_workspace_bytes(ctypes.byref(p))
         if need < 0:
             _lib.check(int(need), "ca_server_forward")
@@ -373,7 +407,7 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
     buffer."""
     dev = recv_buffer.device
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
-    in_place = in_place and (hq * 4) % 16 == 0 and dtype == torch.bfloat16
+    in_place = in_place and (hq * 4) % 16 == 0 and dtype in _ELEM_CODE and d == HEAD_DIM
     # summed dK/dV of shared rows come from float atomics: not when the caller insists on a deterministic backward
     shared = meta.shared_kv if in_place and not fa_args.deterministic else None
     k_rows = shared.num_rows if shared is not None else meta.k_shape[0]
@@ -390,7 +424,7 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
         scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
         lib = _lib.load()
         p = _params(cu_seqlens_q.shape[0] - 1, tq, tk, hq, hkv, d, max_seqlen_q, max_seqlen_kv, scale, fa_args.causal,
-                    fa_args.deterministic)
+                    fa_args.deterministic, dtype)
         need = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
         if need < 0:
             _lib.check(int(need), "ca_server_backward")

@@ -131,8 +131,8 @@ int distca_grad_sum(void *data, int dtype, const int32_t *num_copies,
  * those bounds is dropped (and counted, see distca_ca_schedule_capacity), never
  * executed out of range.
  *
- * Layouts: q,out,dout,dq [total_q, Hq, D] bf16; k,v,dk,dv [total_k, Hkv, D]
- * bf16; lse [Hq, total_q] fp32 natural-log with the scale included;
+ * Layouts: q,out,dout,dq [total_q, Hq, D] 16-bit elements (bf16 or fp16, by
+ * distca_ca_params.dtype); k,v,dk,dv [total_k, Hkv, D] the same; lse [Hq, total_q] fp32 natural-log with the scale included;
  * cu_seqlens_* int32 [B+1]; kv_task_offsets int32 [B] or NULL.
  * D must be 128 in this build.
  *
@@ -152,7 +152,9 @@ typedef struct distca_ca_params {
   int32_t causal;       /* 0 / 1                                              */
   int32_t deterministic;/* backward only: 1 = refuse any path that uses float
                            atomics (only the kv_task_offsets form does)       */
-  int32_t reserved;
+  int32_t dtype;        /* element type of q, k, v, out and the gradients:
+                           DISTCA_DTYPE_BF16 or DISTCA_DTYPE_F16; 0 (callers
+                           written before the field existed) means bf16      */
 } distca_ca_params;
 
 /* Size of the workspace an attention call needs (no reference counterpart: flash-attn
@@ -195,8 +197,8 @@ int distca_ca_fwd_noalloc(const void *q, const void *k, const void *v, void *out
  * receive buffer, runs attention, and packs [out | lse] tokens into the send
  * buffer, attn_kernels/dispatch.py:209-221; here the kernel reads and writes
  * those tokens in place).  Token t of task b of the queries starts at
- * q_base + q_task_off[b] + t * q_tok_bytes and holds Hq*D bf16; of the output at
- * out_base + out_task_off[b] + t * out_tok_bytes and receives Hq*D bf16, then,
+ * q_base + q_task_off[b] + t * q_tok_bytes and holds Hq*D elements; of the output at
+ * out_base + out_task_off[b] + t * out_tok_bytes and receives Hq*D elements, then,
  * when lse is NULL, Hq fp32 lse values and zero padding up to the next multiple
  * of 16 bytes.  A NULL offset array means the packed tensor (offset of task b =
  * cu_seqlens_q[b] tokens, token size Hq*D*2); lse == NULL needs out_task_off.
@@ -228,8 +230,8 @@ int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v,
  * of attn_kernels/dispatch.py:138-206 into four tensors, runs the backward and
  * packs dq; here the kernels read the parts of each token in place and write dq
  * tokens into the send buffer).  Token t of task b of the request starts at
- * req_base + req_task_off[b] + t * req_tok_bytes and holds Hq*D bf16 dO, Hq*D
- * bf16 O, Hq fp32 lse, Hq*D bf16 q; dq token t of task b starts at
+ * req_base + req_task_off[b] + t * req_tok_bytes and holds Hq*D elements of dO, Hq*D
+ * of O, Hq fp32 lse, Hq*D elements of q; dq token t of task b starts at
  * dq_base + dq_task_off[b] + t * dq_tok_bytes.  Needs Hq % 4 == 0 (the q part must
  * stay 16-byte aligned; other head counts return DISTCA_E_UNSUPPORTED and are
  * served by distca_ca_bwd on unpacked tensors).  dk / dv as in distca_ca_bwd. */

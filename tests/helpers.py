@@ -44,14 +44,15 @@ def error_figures(got: torch.Tensor, ref: torch.Tensor) -> dict:
     """Every figure the parity bar is stated in, raw and as asserted:
       max_abs        max |x - ref|                              (raw)
       mre            mean|x - ref| / mean|ref|                  (raw)
-      floor          mre(bf16(ref), ref): what rounding the exact result to bf16 costs
+      floor          mre(round(ref), ref): what rounding the exact result to the output type (bf16; fp16 for fp16 outputs) costs
       max_abs_scaled max |x - ref| / max(1, |ref|)              (asserted <= 2e-2)
       mre_excess     mre - floor                                (asserted <= 1e-3)
       ref_absmax     max |ref|"""
+    out_dtype = got.dtype if got.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
     got = got.detach().float().cpu()
     ref = ref.detach().float().cpu()
     diff = (got - ref).abs()
-    floor = mre(ref.to(torch.bfloat16).float(), ref)
+    floor = mre(ref.to(out_dtype).float(), ref)   # what rounding the exact result to the kernel's output type costs
     raw = mre(got, ref)
     return dict(max_abs=diff.max().item(), mre=raw, floor=floor, max_abs_scaled=(diff / ref.abs().clamp_min(1.0)).max().item(),
                 mre_excess=raw - floor, ref_absmax=ref.abs().max().item(), numel=ref.numel())

@@ -55,13 +55,13 @@ def test_abi_version_and_error_string():
 
 def _p(**kw):
     base = dict(num_tasks=1, total_q=16, total_k=16, num_heads_q=32, num_heads_kv=8, head_dim=128,
-                max_seqlen_q=16, max_seqlen_k=16, softmax_scale=0.088, causal=1, deterministic=0, reserved=0)
+                max_seqlen_q=16, max_seqlen_k=16, softmax_scale=0.088, causal=1, deterministic=0, dtype=0)
     base.update(kw)
     return _lib.CaParams(*[base[f] for f, _ in _lib.CaParams._fields_])
 
 
 @pytest.mark.parametrize("bad", [dict(head_dim=64), dict(num_heads_q=30), dict(num_heads_kv=0), dict(num_tasks=-1),
-                                 dict(total_q=-5)])
+                                 dict(total_q=-5), dict(dtype=3), dict(dtype=-1)])
 def test_unsupported_shapes_are_rejected_on_the_host(bad):
     lib = _lib.load()
     p = _p(**bad)
@@ -74,6 +74,9 @@ def test_unsupported_shapes_are_rejected_on_the_host(bad):
 
 def test_workspace_sizes_are_positive_and_monotone():
     lib = _lib.load()
+    # element type: 0 (callers from before the field existed) and DISTCA_DTYPE_BF16 = 2 mean bf16, 1 is fp16; same sizes
+    sizes = {lib.distca_ca_bwd_workspace_bytes(ctypes.byref(_p(dtype=t))) for t in (0, 1, 2)}
+    assert len(sizes) == 1 and min(sizes) > 0
     small = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(_p()))
     big = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(_p(total_q=131072, total_k=131072, num_tasks=27,
                                                               max_seqlen_q=65536, max_seqlen_k=65536)))

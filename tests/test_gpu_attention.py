@@ -9,12 +9,13 @@ from oracle.attention import ca_reference_bwd, ca_reference_fwd
 pytestmark = pytest.mark.gpu
 
 
-def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128, kv_grad_tol=None):
+def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128, kv_grad_tol=None,
+         dtype=torch.bfloat16):
     from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
     cu_q, cu_k = cu(q_lens), cu(k_lens)
     tq = int(cu_q[-1])
     tk = int(total_k if total_k is not None else cu_k[-1])
-    q, k, v, do = make_qkv(tq, tk, hq, hkv, d, seed)
+    q, k, v, do = (t.to(dtype) for t in make_qkv(tq, tk, hq, hkv, d, seed))   # bf16 values are exact in fp16 at this scale
     ref_out, ref_lse = ca_reference_fwd(q, k, v, cu_q, cu_k, causal=causal, kv_task_offsets=kv_offsets)
     dcu_q = torch.tensor(cu_q, device=cuda)
     dcu_k = torch.tensor(cu_k, device=cuda)
@@ -23,6 +24,7 @@ def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, tota
     print(f"case q_lens={list(q_lens)[:6]} k_lens={list(k_lens)[:6]} hq={hq} hkv={hkv} causal={causal} alias={kv_offsets is not None}", flush=True)
     out, lse = ca_varlen_fwd(qd, kd, vd, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal, dkv)
     torch.cuda.synchronize()
+    assert out.dtype == dtype and out.shape == qd.shape
     assert_close_bf16(out, ref_out, "out")
     finite = torch.isfinite(ref_lse)
     lse_c = lse.cpu()
@@ -36,6 +38,7 @@ def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, tota
     dq, dk, dv = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal,
                                False, dkv)
     torch.cuda.synchronize()
+    assert dq.dtype == dk.dtype == dv.dtype == dtype and dq.shape == qd.shape and dk.shape == kd.shape
     assert_close_bf16(dq, ref_dq, "dq")
     tol = dict(max_abs=kv_grad_tol[0], mean_rel=kv_grad_tol[1]) if kv_grad_tol else {}
     assert_close_bf16(dk, ref_dk, "dk", **tol)
@@ -189,3 +192,60 @@ def test_random_task_batches(cuda, seed):
         return
     k_lens = [q + (int(rng.choice(edges)) if (q and rng.random() < 0.5) else 0) for q in q_lens]
     _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=causal)
+
+
+@pytest.mark.parametrize("case", ["whole", "prefix", "shared", "groups", "pieces"])
+def test_fp16_inputs(cuda, case):
+    """The same kernels compiled for IEEE half precision (the reference's own tests run fp16,
+    tests/test_megatron_layer.py of the reference): whole documents, prefix tasks, tasks that share one stored K/V
+    copy (float atomics in dK/dV), a group of 8 query heads, and a batch small enough for key blocks to be cut into
+    pieces.  Same bar as bf16, with the rounding floor taken in fp16 (its rounding error is an eighth of bf16's, so the
+    bar is the looser of the two here)."""
+    f16 = torch.float16
+    if case == "whole":
+        _run([257, 255, 256, 3, 700], [257, 255, 256, 3, 700], 8, 2, 61, cuda, dtype=f16)
+    elif case == "prefix":
+        _run([128, 200, 64], [384, 200, 1000], 8, 2, 62, cuda, dtype=f16)
+    elif case == "shared":
+        _run([200, 150, 250], [200, 350, 600], 8, 2, 63, cuda, kv_offsets=[0, 0, 0], total_k=600, dtype=f16)
+    elif case == "groups":
+        _run([300, 45], [300, 45], 16, 2, 64, cuda, dtype=f16)
+    else:
+        _run([4096], [4096], 8, 2, 65, cuda, dtype=f16)
+
+
+def test_fp16_and_bf16_agree_on_the_same_values(cuda):
+    """Inputs that are exact in both types give outputs that differ by the types' rounding only: the fp16 build is
+    the bf16 build with another element type, not another algorithm."""
+    from distca_amd.fused_comm_attn import ca_varlen_fwd
+    lens = [513, 64, 300]
+    q, k, v, _ = make_qkv(sum(lens), sum(lens), 8, 2, 128, 66)
+    c = torch.tensor(cu(lens), device=cuda)
+    outs, lses = [], []
+    for dt in (torch.bfloat16, torch.float16):
+        o, l = ca_varlen_fwd(q.to(cuda).to(dt), k.to(cuda).to(dt), v.to(cuda).to(dt), c, c, max(lens), max(lens))
+        outs.append(o.float().cpu()); lses.append(l.cpu())
+    assert (lses[0] - lses[1]).abs().max().item() <= 2e-3
+    assert (outs[0] - outs[1]).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("d,dtype", [(64, torch.bfloat16), (96, torch.float16), (40, torch.bfloat16), (8, torch.bfloat16)])
+def test_head_dims_below_128(cuda, d, dtype):
+    """Head dimensions that are multiples of 8 below 128 (the reference pads to a multiple of 8 and lets flash-attn
+    handle the rest, fused_comm_attn.py:125-129): zero-padded to 128 on the way in, outputs and gradients cut back.
+    The softmax scale is that of the true head dimension."""
+    _run([130, 257, 64], [130, 300, 64], 4, 2, 67 + d, cuda, d=d, dtype=dtype)
+
+
+def test_head_dims_that_are_refused(cuda):
+    from distca_amd.fused_comm_attn import ca_varlen_fwd
+    c = torch.tensor([0, 16], dtype=torch.int32, device=cuda)
+    for d in (136, 256, 100):
+        x = torch.zeros((16, 2, d), dtype=torch.bfloat16, device=cuda)
+        with pytest.raises(RuntimeError, match="head_dim"):
+            ca_varlen_fwd(x, x, x, c, c, 16, 16)
+    q = torch.zeros((16, 2, 128), dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="same for q, k and v"):
+        ca_varlen_fwd(q, q.to(torch.bfloat16), q, c, c, 16, 16)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        ca_varlen_fwd(q.float(), q.float(), q.float(), c, c, 16, 16)

@@ -183,9 +183,11 @@ def test_grad_sum_matches_oracle_on_attention_gradients(cuda):
     assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
 
 
-def test_server_tick_from_single_rank_plan(cuda):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_server_tick_from_single_rank_plan(cuda, dtype):
     """Two documents cut into shards; buffers laid out by metadata.single_rank_plan; the reply of the
-    backward tick, unpacked per stored shard, equals the whole-document gradients."""
+    backward tick, unpacked per stored shard, equals the whole-document gradients.  In both element types of the
+    kernels (in fp16 the in-place ticks read and write the transport tokens in place just the same)."""
     from distca_amd import metadata
     from distca_amd.fused_comm_attn import FlashAttnArgs, ca_server_backward, ca_server_forward
     docs = [[130, 257, 64, 300], [90, 10]]
@@ -193,7 +195,7 @@ def test_server_tick_from_single_rank_plan(cuda):
     fa_params, fmeta, bmeta, (f_recv, f_send, b_recv, b_send) = metadata.server_metas(plan, cuda)
     fa_args = FlashAttnArgs(8, 2, 128)
     T = plan.num_q_tokens
-    q, k, v, do = make_qkv(T, T, 8, 2, 128, 33)
+    q, k, v, do = (t.to(dtype) for t in make_qkv(T, T, 8, 2, 128, 33))
     as_bytes = lambda x: x.reshape(x.shape[0], -1).contiguous().view(torch.uint8).numpy()
     stored = plan.stored_shard_tokens.numpy()
     first_entry = [plan.kv_entry_shard.tolist().index(s) for s in range(len(stored))]
@@ -205,9 +207,9 @@ def test_server_tick_from_single_rank_plan(cuda):
     fa2a.copy_non_cp(as_bytes(v), recv, v_off.numpy()[first_entry], stored)
     send = torch.zeros(f_send, dtype=torch.uint8, device=cuda)
     print("plan forward", flush=True)
-    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args, in_place=False)
+    out, lse = ca_server_forward(torch.from_numpy(recv).to(cuda), send, fmeta, fa_params, fa_args, dtype, in_place=False)
     send_in_place = torch.zeros_like(send)
-    ca_server_forward(torch.from_numpy(recv).to(cuda), send_in_place, fmeta, fa_params, fa_args)
+    ca_server_forward(torch.from_numpy(recv).to(cuda), send_in_place, fmeta, fa_params, fa_args, dtype)
     torch.cuda.synchronize()
     assert torch.equal(send_in_place, send)
     cu_doc = np.concatenate([[0], np.cumsum([sum(d) for d in docs])]).astype(np.int32)
@@ -234,11 +236,11 @@ def test_server_tick_from_single_rank_plan(cuda):
     gsend = torch.zeros(b_send, dtype=torch.uint8, device=cuda)
     print("plan backward", flush=True)
     got = ca_server_backward(torch.from_numpy(recv).to(cuda), gsend, bmeta, fa_args, fa_params.cu_seqlens_q,
-                             fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
+                             fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, dtype)
     assert got[0] is None, "8 query heads: the kernels read the request and write dq in place"
     gsend_steps = torch.zeros_like(gsend)
     ca_server_backward(torch.from_numpy(recv).to(cuda), gsend_steps, bmeta, fa_args, fa_params.cu_seqlens_q,
-                       fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, in_place=False)
+                       fa_params.cu_seqlens_kv, fa_params.max_seqlen_q, fa_params.max_seqlen_kv, dtype, in_place=False)
     torch.cuda.synchronize()
     assert torch.equal(gsend, gsend_steps), "in-place and step-by-step ticks leave the same bytes"
     gq_off, gk_off, gv_off, _ = plan.reply_layout(True)
@@ -247,7 +249,7 @@ def test_server_tick_from_single_rank_plan(cuda):
     fa2a.copy_non_cp(dq, g, gq_off.numpy(), plan.q_seqlens.numpy(), None, False)
     fa2a.copy_non_cp(dk, g, gk_off.numpy()[first_entry], stored, None, False)
     fa2a.copy_non_cp(dv, g, gv_off.numpy()[first_entry], stored, None, False)
-    tb = lambda a, h: torch.from_numpy(a).view(torch.bfloat16).reshape(T, h, 128)
+    tb = lambda a, h: torch.from_numpy(a).view(dtype).reshape(T, h, 128)
     ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_doc, cu_doc, out=out.cpu().reshape(T, 8, 128), softmax_lse=lse.cpu())
     assert_close_bf16(tb(dq, 8), ref_dq, "dq")
     # a stored shard's gradient is the bf16 sum of up to four per-task bf16 gradients: 4e-2 / 3e-3
