@@ -578,6 +578,50 @@ class FusedCommAttn(torch.autograd.Function):
         return (torch.empty((1,), device=signal_grad.device, dtype=signal_grad.dtype),) + (None,) * 8
 
 
+@torch.no_grad()
+def dummy_backward_single_sided(config, packed_seq_params, dtype: torch.dtype, device, attn_out_grad_all2all: bool = True,
+                                qkv_grad_all2all: bool = True):
+    """The backward of FusedCommAttn with its two all-to-alls, outside autograd (fused_comm_attn.py:529-642 of the
+    reference, which a pipeline stage runs for micro-batches whose forward ran elsewhere): the request all-to-all (unless
+    the caller has done it), the server's backward tick, the gradient all-to-all (or, left to the caller, an event
+    recorded behind the tick).  `config` gives num_attention_heads, num_query_groups, hidden_size and
+    tensor_model_parallel_size; buffers are those of dispatcher `packed_seq_params.dispatcher_id`."""
+    from .ops import fast_a2a
+    assert packed_seq_params.bwd_packed_seq_params is not None
+    tp = config.tensor_model_parallel_size
+    num_heads = config.num_attention_heads // tp
+    hidden = config.hidden_size // tp
+    fa_args = FlashAttnArgs(num_heads_q=num_heads, num_heads_kv=config.num_query_groups // tp, head_dim=hidden // num_heads,
+                            return_attn_probs=True)
+    dispatcher_id = packed_seq_params.dispatcher_id
+    req, grad = packed_seq_params.attn_out_bwd_metadata, packed_seq_params.qkv_bwd_metadata
+    stream = getattr(packed_seq_params, "stream", None)
+    if attn_out_grad_all2all:
+        with torch.cuda.stream(stream):
+            fast_a2a(*req.fa2a_metadata, req.my_rank_send_offset, req.my_rank_recv_offset, req.my_rank_send_sz,
+                     instance_id=dispatcher_id)
+        if stream is not None:
+            torch.cuda.current_stream().wait_stream(stream)
+    else:
+        assert dispatcher_id is not None
+    recv_buffer, send_buffer = _server_buffers(dispatcher_id)
+    fused_comm_attn_backward(recv_buffer, send_buffer, packed_seq_params, fa_args, dtype)
+    _server_done(dispatcher_id)
+    if not qkv_grad_all2all:
+        assert dispatcher_id is not None
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream())
+        return event
+    if stream is not None:
+        stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        fast_a2a(*grad.fa2a_metadata, grad.my_rank_send_offset, grad.my_rank_recv_offset, grad.my_rank_send_sz,
+                 instance_id=dispatcher_id)
+    if dispatcher_id is None:
+        DispatcherWrapper.switch_buffer()
+    return None
+
+
 def post_a2a_attn_out_with_lse(recv_buffer: Optional[Tensor], q: Tensor, num_heads_q: int, metadata, dtype: torch.dtype = None,
                                instance_id: int = None, switch_buffer: bool = False):
     """Linear side, forward of the reference's autograd function of the same name

@@ -573,6 +573,24 @@ def test_fused_comm_attn_autograd_function(cuda):
     assert_close_bf16(dq.reshape(T, hq, d), ref_dq, "dq")
     assert_close_bf16(dk_planes.sum(0).reshape(T, hkv, d), ref_dk, "dk", max_abs=4e-2, mean_rel=3e-3)
     assert_close_bf16(dv_planes.sum(0).reshape(T, hkv, d), ref_dv, "dv", max_abs=4e-2, mean_rel=3e-3)
+    # the same backward outside autograd, all-to-alls included (what a pipeline stage runs for foreign micro-batches)
+    from types import SimpleNamespace
+    from distca_amd.fused_comm_attn import dummy_backward_single_sided
+    post_a2a_attn_out_with_lse_backward(None, dod, attn_out, lse_bytes.contiguous(), qd, kd, vd, req, instance_id=ID)
+    step.dispatcher_id = ID
+    config = SimpleNamespace(num_attention_heads=hq, num_query_groups=hkv, hidden_size=hq * d, tensor_model_parallel_size=1)
+    print("dummy_backward_single_sided", flush=True)
+    assert dummy_backward_single_sided(config, step, torch.bfloat16, cuda) is None
+    assert DispatcherWrapper.is_acquired[ID], "the gradient all-to-all has filled the receive buffer"
+    off = int(grad.my_rank_recv_offset)
+    assert torch.equal(recv_of()[off:off + n], explicit_grads)
+    DispatcherWrapper.release(ID)
+    post_a2a_attn_out_with_lse_backward(None, dod, attn_out, lse_bytes.contiguous(), qd, kd, vd, req, instance_id=ID)
+    a2a(req)
+    event = dummy_backward_single_sided(config, step, torch.bfloat16, cuda, attn_out_grad_all2all=False, qkv_grad_all2all=False)
+    assert isinstance(event, torch.cuda.Event) and not DispatcherWrapper.is_acquired[ID]
+    event.synchronize()
+    assert torch.equal(send_of()[:n], explicit_grads)
     # without an instance id the ticks alternate between the two instances
     DispatcherWrapper.cur_instance = 0
     from distca_amd.fused_comm_attn import _server_buffers
