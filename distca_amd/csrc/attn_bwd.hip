@@ -10,23 +10,8 @@
 // (row, key) pair per 128 keys, 124 GB at 128K tokens) took as long as the rest of the kernel.
 //
 //   1. bwd_prepare_kernel: per (token, head) row, scale*<dO, O> and lse*log2(e) -> workspace.
-//   2. ca_bwd_dkdv_kernel: one workgroup of 8 waves per (task, block of 256 keys, kv head),
-//      in the order of the backward tile schedule.  V of the block sits in LDS for the
-//      workgroup's life, K in registers (each wave's 32 keys as B operand; the waves form two
-//      groups of four, group 0 with the block's first 128 keys, group 1 with the rest).  The
-//      query side (Q, dO and the two row statistics of every head of the kv group, flattened into
-//      rows like the forward) is streamed in blocks of 32 rows from the first block the causal
-//      mask lets see these keys; both groups work through every block, half a period apart, so
-//      that every SIMD holds two waves at different points of the loop body and a block is
-//      fetched once for 256 keys.  Per block and wave:
-//        S = Q K^T, dP = dO V^T            A from the query tile, B = K registers / V tile (LDS)
-//        P = exp2(S*c - lse2), dS / scale = P (dP - delta)              in registers
-//        dV^T += dO^T P, dK^T += Q^T dS    A by transposing LDS reads of the same query tile,
-//                                          B = the accumulator registers converted to bf16
-//      Query tiles arrive two periods ahead through LDS-direct global loads (each wave brings
-//      four 256-byte rows of Q and of dO per tile, one instruction each) into a ring of four
-//      stages; the tile has unpadded rows whose 16-byte chunks are swizzled (tile_swz), which
-//      serves both read shapes without bank conflicts.
+//   2. ca_bwd_dkdv64_kernel (attn_bwd_dkdv64.hip): dK and dV, one workgroup of 4 waves per (task, block of
+//      256 keys, kv head), in the order of the backward tile schedule.
 //   3. ca_bwd_dq_kernel: one workgroup of 8 waves per (task, block of 256 flattened query
 //      rows, kv head), in the order of the forward tile schedule; the mirror image of the
 //      forward kernel.  Q and dO stay in registers as B operands, K/V tiles of 64 keys are
@@ -46,409 +31,7 @@
 namespace distca {
 namespace {
 
-#ifndef DISTCA_DKDV64
-#define DISTCA_DKDV64 1
-#endif
-constexpr int kPitch = 272;  // bytes per 128-element bf16 row in LDS
 constexpr float kLog2e = 1.4426950408889634f;
-
-// ------------------------------------------------------------------------------------------
-// dK / dV
-// ------------------------------------------------------------------------------------------
-constexpr int kBwdThreads = 512;
-constexpr int kBN = kBwdKV;    // 256 keys per workgroup
-constexpr int kBM = kBwdRows;  // 32 flattened query rows per block
-
-// LDS map (bytes): V of the block for the workgroup's life; behind it a region that first stages K on
-// its way into registers and then holds the ring of query-side tiles
-constexpr int kVsOff = 0;
-constexpr int kKsOff = kVsOff + kBN * kPitch;
-constexpr int kTileOff = kKsOff;
-constexpr int kTileRow = 256;                     // query-side tiles: unpadded rows, swizzled chunks (tile_swz)
-constexpr int kTileQ = 0, kTileDO = kBM * kTileRow;
-constexpr int kTileBytes = 2 * kBM * kTileRow;    // Q + dO of one block
-constexpr int kStages = 4;                        // a tile is requested two periods ahead and read for a period and a half
-constexpr int kStatOff = kTileOff + kStages * kTileBytes;
-constexpr int kStatBytes = 3 * kBM * 4;           // per stage: lse2, dscaled, lim
-constexpr int kBwdLds = kKsOff + kBN * kPitch;
-static_assert(kStatOff + kStages * kStatBytes <= kBwdLds, "tile ring must fit in the K staging region");
-static_assert(kBwdLds <= 160 * 1024, "LDS budget");
-
-template <bool ALIAS>
-__global__ __launch_bounds__(kBwdThreads, 1) void ca_bwd_dkdv_kernel(BwdArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  const int nitems = a.sched[0];
-  int item, kvh;
-  if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
-  const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
-  const int task = it4.x, nblk = it4.y;
-
-  const int q0 = a.cu_q[task];
-  const int lq = a.cu_q[task + 1] - q0;
-  const int lk = a.cu_k[task + 1] - a.cu_k[task];
-  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
-  const int G = a.group;
-  const int shift = lk - lq;
-  const int nrows = lq * G;
-  const int nmb = (nrows + kBM - 1) / kBM;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be so
-  const int grp = wave >> 2, kbw = wave & 3;
-  const int l32 = lane & 31, g = lane >> 5;
-  const int kb0 = nblk * kBN;      // first key of the workgroup
-  const int kw0 = kb0 + (grp * 4 + kbw) * 32;  // first key of the wave: group 0 the block's first 128 keys, group 1 the rest
-
-  int mb0 = 0;
-  if (a.causal) {
-    int t_first = kb0 - shift;
-    if (t_first < 0) t_first = 0;
-    mb0 = (int)(((int64_t)t_first * G) / kBM);
-  }
-  // the query blocks of this item, visited from block top - 1 down to block bot: all that see the key block,
-  // or one piece of them (sched.h)
-  int top = nmb, bot = mb0;
-  {
-    const int piece = it4.w & 0xffff, pieces = it4.w >> 16;
-    if (pieces > 1) {
-      const int n = nmb > mb0 ? nmb - mb0 : 0;
-      top = nmb - piece_begin(n, piece, pieces);
-      bot = nmb - piece_begin(n, piece + 1, pieces);
-    }
-  }
-  const int niter = top > bot ? top - bot : 0;
-
-  const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
-
-  // ---- K and V of the block into LDS (rows past the prefix as zeros)
-  {
-    const int col = tid & 15, row = tid >> 4;  // 32 rows per pass
-#pragma unroll
-    for (int i = 0; i < kBN / 32; ++i) {
-      const int r = row + 32 * i;
-      const int key = kb0 + r;
-      u32x4 kv = u32x4{0, 0, 0, 0}, vv = u32x4{0, 0, 0, 0};
-      if (key < lk) {
-        const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim + col * 8;
-        kv = *reinterpret_cast<const u32x4 *>(a.k + off);
-        vv = *reinterpret_cast<const u32x4 *>(a.v + off);
-      }
-      *reinterpret_cast<u32x4 *>(lds + kKsOff + r * kPitch + col * 16) = kv;
-      *reinterpret_cast<u32x4 *>(lds + kVsOff + r * kPitch + col * 16) = vv;
-    }
-  }
-
-  f32x16 dkacc[4], dvacc[4];
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      dkacc[db][r] = 0.f;
-      dvacc[db][r] = 0.f;
-    }
-
-  // byte offset of (token 0 of the task, first head of the group) in the query-side region
-  const int64_t qbase = (a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes) + (int64_t)kvh * G * kHeadDim * 2;
-
-  // ---- query-side tile fetch: this wave brings rows 8*kbw .. 8*kbw+7 of its group's block.
-  // Rows past the task (and a group's last block when it does not exist) are clamped to the
-  // task's last row so that the loads stay in bounds, and marked by lim = -1 (every key masked).
-  auto div_group = [&](int n) { return a.group_magic ? (int)__umulhi((uint32_t)n, a.group_magic) : n; };
-  // The fetch of one block in three pieces: row statistics, rows 0-3, rows 4-7 of this wave's share.
-  // (Issuing them between the MFMAs of phase A, as the forward kernel does, measured 2 % slower here:
-  // the other group is in its LDS-bound phase C at that time.)
-  // Blocks whose 32 rows all exist take a form without per-lane address arithmetic when the group size
-  // divides 32 (a block then starts at a token boundary): scalar bases that move by one block, plus per-lane
-  // offsets that never change.
-  const bool fast_ok = (kBM % G) == 0 && (int64_t)G * a.total_q * 4 < (1ll << 32) && 32 * a.qs_tok_bytes < (1ll << 32);
-  const int tok_per_blk = kBM / G;
-  uint32_t voff_q, voff_s;
-  int tok_s;
-  {
-    const int rl = wave * 4 + (lane >> 4);
-    const int tq = div_group(rl);
-    voff_q = (uint32_t)(tq * a.qs_tok_bytes + (rl - tq * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(rl)) << 4));
-    const int rs = wave * 4 + (lane & 3);
-    tok_s = div_group(rs);
-    voff_s = (uint32_t)((((int64_t)(rs - tok_s * G)) * a.total_q + tok_s) * 4);
-  }
-  const float *stat_base = a.lse2 + (int64_t)kvh * G * a.total_q + q0;
-  const int64_t stat_delta = a.dscaled - a.lse2;
-  auto issue_tile = [&](int stage, int mbx) {
-    const int tile = kTileOff + stage * kTileBytes;
-    const int stat = kStatOff + stage * kStatBytes;
-    const bool blk_ok = mbx >= bot;
-    if (fast_ok && blk_ok && (mbx + 1) * kBM <= nrows) {
-      const int tok0 = mbx * tok_per_blk;
-      if (lane < 4) {
-        int lm = a.causal ? tok0 + tok_s + shift : lk - 1;
-        if (lm > lk - 1) lm = lk - 1;
-        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[wave * 4 + lane] = lm;
-        lds_direct_load4_base(stat_base + tok0, voff_s, lds0 + stat + wave * 16);
-        lds_direct_load4_base(stat_base + stat_delta + tok0, voff_s, lds0 + stat + kBM * 4 + wave * 16);
-      }
-      const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
-      const uint8_t *db = reinterpret_cast<const uint8_t *>(a.dout) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
-      const uint32_t dst = lds0 + tile + wave * 4 * kTileRow;
-      lds_direct_load16(qb, voff_q, dst + kTileQ);
-      lds_direct_load16(db, voff_q, dst + kTileDO);
-      return;
-    }
-    {  // row statistics: lanes 0..3 take one of the wave's four rows each
-      const int rl = wave * 4 + (lane & 3);
-      const int rho = mbx * kBM + rl;
-      const bool ok = blk_ok && rho < nrows;
-      const int rc = ok ? rho : nrows - 1;
-      const int tok = div_group(rc);
-      const int hg = rc - tok * G;
-      if (lane < 4) {
-        int lm = a.causal ? tok + shift : lk - 1;
-        if (lm > lk - 1) lm = lk - 1;
-        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
-        const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
-        lds_direct_load4(a.lse2 + so, lds0 + stat + wave * 16);
-        lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + wave * 16);
-      }
-    }
-    {  // Q and dO: one instruction fills the wave's four rows; lane p brings the chunk that belongs at
-       // chunk position p%16 of row p/16.  Rows that do not exist read the zero row.
-      const int rl = wave * 4 + (lane >> 4);
-      const int rho = mbx * kBM + rl;
-      const bool ok = blk_ok && rho < nrows;
-      const int tok = div_group(ok ? rho : 0);
-      const int hg = (ok ? rho : 0) - tok * G;
-      const int chunk = (lane & 15) ^ tile_swz(rl);
-      const int64_t eo = qbase + (int64_t)tok * a.qs_tok_bytes + hg * (kHeadDim * 2);
-      const elem_t *qs = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.q) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
-      const elem_t *ds = reinterpret_cast<const elem_t *>(ok ? reinterpret_cast<const uint8_t *>(a.dout) + eo : reinterpret_cast<const uint8_t *>(a.zero_row));
-      const uint32_t dst = lds0 + tile + wave * 4 * kTileRow;
-      lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
-      lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
-    }
-  };
-  // a wave has four fetch instructions per tile; older tiles have landed once at most that many are pending
-  auto wait_older = [&]() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); };
-
-  const float c = a.scale * kLog2e;
-  // tile-independent LDS offsets
-  const int a_rd = l32 * kTileRow + ((g ^ tile_swz(l32)) << 4);  // A operand rows of the query tile, ^ 32*s
-  const int b_rd = ((grp * 4 + kbw) * 32 + l32) * kPitch + 16 * g;  // B operand rows of K / V, + 32*s
-  // transposed A operand: lane points at (row 4g + i4 [+8 hi +16 (j>>2)], chunk 8 b4 + h1 [+2 (j&3)], half lane&1);
-  // tile_swz of that row is (i4<<1) | (g<<3) | hi
-  const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
-  const int t_rd = (4 * g + i4) * kTileRow + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*(j&3) ^ 16*hi
-
-  elemx8 kreg[8];  // this wave's 32 keys as B operand of S = Q K^T, all 8 steps over d
-  f32x16 sacc, dpacc;
-  // ---- phase A: S = Q K^T, dP = dO V^T   (rows: queries, cols: this wave's keys) -- MFMA only
-  auto phase_a = [&](int stage) {
-    const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
-    // dP accumulates on top of -delta of its rows (register r of the accumulator is query row 8 (r / 4) + 4 g + r % 4),
-    // so that phase B has dP - delta without an instruction; the scale is applied to dK once, at the end
-    const uint8_t *stat_a = lds + kStatOff + stage * kStatBytes + kBM * 4;
-#pragma unroll
-    for (int cq = 0; cq < 4; ++cq) {
-      const f32x4 nd = *reinterpret_cast<const f32x4 *>(stat_a + (8 * cq + 4 * g) * 4);
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) dpacc[4 * cq + rr] = nd[rr];
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-    // operands of step s+1 are requested before the MFMAs of step s are issued
-    constexpr int kDa = 2;  // operand fetch distance in MFMA steps
-    elemx8 qa[kDa], da[kDa], vb[kDa];
-    auto load_a = [&](int s, int buf) {
-      const int ao = a_rd ^ (s << 5);
-      qa[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileQ + ao);
-      da[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileDO + ao);
-      vb[buf] = *reinterpret_cast<const elemx8 *>(lds + kVsOff + b_rd + 32 * s);
-    };
-#pragma unroll
-    for (int s = 0; s < kDa; ++s) load_a(s, s);
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      __builtin_amdgcn_sched_barrier(0);
-      sacc = mfma32(qa[s % kDa], kreg[s], sacc);
-      dpacc = mfma32(da[s % kDa], vb[s % kDa], dpacc);
-      __builtin_amdgcn_sched_barrier(0);
-      if (s + kDa < 8) load_a(s + kDa, s % kDa);
-    }
-  };
-  // ---- phase B (VALU): P and dS, converted to bf16 B operands
-  elemx8 pb[2], dsb[2];
-  auto phase_b = [&](int stage) {
-    const uint8_t *stat = lds + kStatOff + stage * kStatBytes;
-    const int lim_first = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[0];
-    const int lim_last = reinterpret_cast<const int *>(stat + 2 * kBM * 4)[kBM - 1];
-    const bool need_mask = (kw0 + 31 > lim_first) || (lim_last < 0);
-    // the masked form only for tiles that straddle the diagonal or the end of the task (uniform branch):
-    // compare and select per element are a third of this phase's instructions
-    auto body = [&](auto masked) __attribute__((always_inline)) {
-#pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const int qr = 8 * cq + 4 * g;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
-        i32x4 lim4 = {0x7fffffff, 0x7fffffff, 0x7fffffff, 0x7fffffff};
-        if constexpr (decltype(masked)::value) lim4 = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int r = 4 * cq + rr;
-          float p = fast_exp2(__builtin_fmaf(sacc[r], c, -lse4[rr]));
-          if constexpr (decltype(masked)::value) {
-            if (kw0 + l32 > lim4[rr]) p = 0.f;
-          }
-          const float ds = p * dpacc[r];
-          sacc[r] = p;
-          dpacc[r] = ds;
-        }
-        if (cq == 1) __builtin_amdgcn_sched_barrier(0);  // at most half of the row statistics in registers at a time
-      }
-    };
-    if (need_mask) body(std::true_type{});
-    else body(std::false_type{});
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int r0 = 8 * t;
-      pb[t] = cvt8(sacc[r0], sacc[r0 + 1], sacc[r0 + 2], sacc[r0 + 3], sacc[r0 + 4], sacc[r0 + 5], sacc[r0 + 6], sacc[r0 + 7]);
-      dsb[t] = cvt8(dpacc[r0], dpacc[r0 + 1], dpacc[r0 + 2], dpacc[r0 + 3], dpacc[r0 + 4], dpacc[r0 + 5], dpacc[r0 + 6], dpacc[r0 + 7]);
-    }
-  };
-  // ---- phase C (MFMA): dV^T += dO^T P, dK^T += Q^T dS
-  auto phase_c = [&](int stage) {
-    const uint8_t *tile = lds + kTileOff + stage * kTileBytes;
-    constexpr int kDc = 2;  // operand fetch distance in MFMA steps
-    elemx4 ct[kDc][4];  // [buffer][dO^T lo, dO^T hi, Q^T lo, Q^T hi]
-    auto load_c = [&](int j, int buf) {
-      const int lo = (16 * (j >> 2)) * kTileRow + (t_rd ^ ((j & 3) << 5));
-      const int hi = (16 * (j >> 2) + 8) * kTileRow + (t_rd ^ ((j & 3) << 5) ^ 16);
-      ct[buf][0] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + lo));
-      ct[buf][1] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileDO + hi));
-      ct[buf][2] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + lo));
-      ct[buf][3] = lds_read_tr((const DISTCA_LDS void *)(tile + kTileQ + hi));
-    };
-#pragma unroll
-    for (int j = 0; j < kDc; ++j) load_c(j, j);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      __builtin_amdgcn_sched_barrier(0);
-      dvacc[j & 3] = mfma32(cat4(ct[j % kDc][0], ct[j % kDc][1]), pb[j >> 2], dvacc[j & 3]);
-      dkacc[j & 3] = mfma32(cat4(ct[j % kDc][2], ct[j % kDc][3]), dsb[j >> 2], dkacc[j & 3]);
-      __builtin_amdgcn_sched_barrier(0);
-      if (j + kDc < 8) load_c(j + kDc, j % kDc);
-    }
-  };
-
-  // Both groups work through every tile, half a period apart: between barriers b1(p) and b2(p) group 0
-  // is in its MFMA-only phase A of tile p while group 1 does the arithmetic phase B and then phase C of
-  // tile p-1; after b2(p) the roles swap.  A SIMD holds one wave of each group, so its MFMA pipe and its
-  // VALU are busy at the same time instead of by turns.
-  //   [b1(p), b2(p)):    g0: fetch(p+2), A(p)     g1: B(p-1), C(p-1)
-  //   [b2(p), b1(p+1)):  g0: B(p), C(p)           g1: fetch(p+2), A(p)
-  // (Moving B in front of b2, which evens out the instruction counts of the two halves, measured 14 %
-  // slower: phases A and C both live on LDS reads and then run together.)
-  // Tile p is read from b1(p) to b2(p+1).  Every wave requests its four rows of tile p+2 at the start of
-  // its phase A of tile p, into the stage tile p-2 left at b2(p-1), and makes sure before each b1 that at
-  // most its newest request is pending, so that tile p is complete at b1(p).  Requests are made for
-  // tiles past the end as well (their rows come from the zero row), which keeps that count fixed.
-  // A wave raises its priority for its MFMA phases: the instruction arbiter prefers the older wave
-  // of a SIMD, which otherwise lets group 0's arithmetic phase hold up group 1's MFMAs (-1.3 %).
-  // Each group has its own copy of the loop (every wave passes the same 2*niter + 1 barriers), which
-  // keeps the register allocation of either path as small as a single loop's.
-  // Blocks are visited from the last one down to the diagonal: workgroups that run at the
-  // same time (neighbouring key blocks of one document, by the schedule) then read the same
-  // query rows at the same time and find them in their XCD's L2.
-  __syncthreads();
-#pragma unroll
-  for (int s = 0; s < 8; ++s) kreg[s] = *reinterpret_cast<const elemx8 *>(lds + kKsOff + b_rd + 32 * s);
-  __syncthreads();  // K has left LDS: its region now holds the tile ring
-  if (niter > 0) {
-    issue_tile(0, top - 1);
-    issue_tile(1, top - 2);
-  }
-  wait_vm0();
-  if (grp == 0) {
-    for (int p = 0; p < niter; ++p) {
-      wait_older();
-      __syncthreads();  // b1(p): tile p is complete
-      issue_tile((p + 2) % kStages, top - 1 - (p + 2));
-      __builtin_amdgcn_s_setprio(3);
-      phase_a(p % kStages);
-      __builtin_amdgcn_s_setprio(0);
-      __syncthreads();  // b2(p)
-      phase_b(p % kStages);
-      __builtin_amdgcn_s_setprio(3);
-      phase_c(p % kStages);
-      __builtin_amdgcn_s_setprio(0);
-    }
-    __syncthreads();  // b1(niter), which group 1 passes between its last phases A and B
-  } else {
-    __syncthreads();    // b1(0)
-    for (int p = 0; p < niter; ++p) {
-      __syncthreads();  // b2(p)
-      issue_tile((p + 2) % kStages, top - 1 - (p + 2));
-      __builtin_amdgcn_s_setprio(3);
-      phase_a(p % kStages);
-      __builtin_amdgcn_s_setprio(0);
-      wait_older();
-      __syncthreads();  // b1(p+1): tile p+1 is complete
-      phase_b(p % kStages);
-      __builtin_amdgcn_s_setprio(3);
-      phase_c(p % kStages);
-      __builtin_amdgcn_s_setprio(0);
-    }
-  }
-  wait_vm0();  // nothing may still be on its way into LDS when the workgroup ends
-
-  // ---- epilogue: dK, dV of this wave's keys (registers 4*cq..+3 of block db hold d0..d0+3)
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dkacc[db][r] *= a.scale;
-  if (ALIAS) {
-    // Work items that share K/V rows (tasks over one stored prefix, pieces of one key block) add up in
-    // fp32; the order of these additions is the one source of run-to-run variation.  A lane holds one key's
-    // values, 2 KB apart from its neighbour's in memory: the sums pass through LDS so that one atomic
-    // instruction covers 64 consecutive floats of a row instead of 64 rows.
-    constexpr int kEpiPitch = (kHeadDim + 4) * 4;  // bytes per key row in LDS; the 16 spare bytes spread the banks
-    static_assert(kBN * kEpiPitch <= kBwdLds, "the epilogue stages one 256 x 128 fp32 matrix in LDS");
-    const int wkey0 = (grp * 4 + kbw) * 32;        // this wave's rows of the staging matrix: written and read by it alone
-    const int nkeys = lk - kw0 < 32 ? lk - kw0 : 32;
-    __syncthreads();                               // every wave has finished with the V tile and the tile ring
-#pragma unroll
-    for (int which = 0; which < 2; ++which) {
-      float *dst = which == 0 ? a.dk_acc : a.dv_acc;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int cq = 0; cq < 4; ++cq) {
-          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          const f32x16 &acc = which == 0 ? dkacc[db] : dvacc[db];
-          *reinterpret_cast<f32x4 *>(lds + (wkey0 + l32) * kEpiPitch + d0 * 4) = f32x4{acc[4 * cq], acc[4 * cq + 1], acc[4 * cq + 2], acc[4 * cq + 3]};
-        }
-      // LDS operations of one wave complete in order: the reads below see the writes above
-      for (int kk = 0; kk < nkeys; ++kk) {
-        const float *row = reinterpret_cast<const float *>(lds + (wkey0 + kk) * kEpiPitch);
-        float *out = dst + (int64_t)(ks + kw0 + kk) * kv_stride + kvh * kHeadDim;
-        unsafeAtomicAdd(out + lane, row[lane]);
-        unsafeAtomicAdd(out + 64 + lane, row[64 + lane]);
-      }
-    }
-  } else {
-    const int key = kw0 + l32;
-    if (key < lk) {
-      const int64_t off = (int64_t)(ks + key) * kv_stride + kvh * kHeadDim;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int cq = 0; cq < 4; ++cq) {
-          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          *reinterpret_cast<elemx4 *>(a.dk + off + d0) = cvt4(dkacc[db][4 * cq], dkacc[db][4 * cq + 1], dkacc[db][4 * cq + 2], dkacc[db][4 * cq + 3]);
-          *reinterpret_cast<elemx4 *>(a.dv + off + d0) = cvt4(dvacc[db][4 * cq], dvacc[db][4 * cq + 1], dvacc[db][4 * cq + 2], dvacc[db][4 * cq + 3]);
-        }
-    }
-  }
-}
 
 // ------------------------------------------------------------------------------------------
 // dQ
@@ -951,10 +534,8 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: max_seqlen_q * (Hq/Hkv)^2 must stay below 2^32");
 
   if (device_setup_pending(kSlotBwdLds)) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipError_t e3 = hipFuncSetAttribute((const void *)ca_bwd_dq_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
-    if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve LDS");
+    hipError_t e = hipFuncSetAttribute((const void *)ca_bwd_dq_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
+    if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS: %s", kDqLds, hipGetErrorString(e));
     device_setup_done(kSlotBwdLds);
   }
 
@@ -973,15 +554,8 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
-#if DISTCA_DKDV64
     rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, s);
     if (rc) return rc;
-#else
-    if (use_acc)
-      hipLaunchKernelGGL((ca_bwd_dkdv_kernel<true>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
-    else
-      hipLaunchKernelGGL((ca_bwd_dkdv_kernel<false>), dim3((unsigned)grid), dim3(kBwdThreads), kBwdLds, s, a);
-#endif
   }
   // ---- dQ: one workgroup per (task, block of query rows, kv head)
   {

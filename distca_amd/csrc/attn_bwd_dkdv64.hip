@@ -18,7 +18,7 @@
 //   step 4   dK^T += Q^T dS    16 MFMAs   A: transposing reads of the Q tile, B: dS
 //
 // Every LDS fragment a wave reads feeds two MFMAs (one per key block of the wave): half the LDS traffic per MFMA of
-// a 32-key wave, which is what bounded the eight-wave form of this kernel.
+// a 32-key wave: with eight waves of 32 keys, two per SIMD, the LDS reads bounded the kernel.
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 #include "api_util.h"

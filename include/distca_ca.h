@@ -282,7 +282,7 @@ int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
  * and clears them.  Not thread safe; leave disabled outside benchmarks.
  * ------------------------------------------------------------------------- */
 #define DISTCA_TIMER_CA_FWD 0      /* ca_fwd_kernel                          */
-#define DISTCA_TIMER_CA_BWD 1      /* ca_bwd_dkdv_kernel                     */
+#define DISTCA_TIMER_CA_BWD 1      /* ca_bwd_dkdv64_kernel                   */
 #define DISTCA_TIMER_MEMCPY_NON_CP 2
 #define DISTCA_TIMER_MEMCPY_CP 3
 #define DISTCA_TIMER_GRAD_SUM 4
