@@ -48,7 +48,7 @@ static_assert(kLds <= 160 * 1024, "LDS budget");
 #ifndef DISTCA_RAWBAR
 #define DISTCA_RAWBAR 1
 #endif
-constexpr int kLoadsPerBlock = 6;        // vector-memory instructions a wave issues per block
+constexpr int kLoadsPerBlock = 5;        // vector-memory instructions a wave issues per block
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <int N>
@@ -152,15 +152,19 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   // byte offset of (token 0 of the task, first head of the group) in the query-side region
   const int64_t qbase = (a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes) + (int64_t)kvh * G * kHeadDim * 2;
 
-  // ---- query-side tile fetch: this wave brings rows 8 w .. 8 w + 7 of a block (kLoadsPerBlock vector-memory
-  // instructions: two for the row statistics, two each for its rows of Q and of dO).  Rows that do not exist
-  // (past the task, or a block below the item's last) read the zero row and get lim = -1 (every key masked).
-  // Blocks whose 32 rows all exist take a form without per-lane address arithmetic when the group size divides 32
-  // (a block then starts at a token boundary): scalar bases that move by one block, per-lane offsets that never change.
-  const bool fast_ok = (kBM % G) == 0 && (int64_t)G * a.total_q * 4 < (1ll << 32) && 32 * a.qs_tok_bytes < (1ll << 32);
+  // ---- query-side tile fetch: this wave brings rows 8 w .. 8 w + 7 of a block, two LDS-direct loads each for its
+  // rows of Q and of dO, and (every wave, to the same place) the 64 row statistics of the block with one load: lane L
+  // fetches lse2 of row L % 32 for L < 32 and -delta of that row for L >= 32, which is the order they have in LDS.
+  // kLoadsPerBlock vector-memory instructions per wave and block in every form, which the counted waits rely on.
+  // Rows that do not exist (past the task, or a block below the item's last) read the zero row and get lim = -1
+  // (every key masked).  Blocks whose 32 rows all exist take a form without per-lane address arithmetic when the
+  // group size divides 32 (a block then starts at a token boundary): scalar bases, per-lane offsets that never change.
+  const float *stat_lo = a.lse2 < a.dscaled ? a.lse2 : a.dscaled;  // the two arrays lie in one workspace
+  const int64_t stat_span = a.lse2 < a.dscaled ? a.dscaled - a.lse2 : a.lse2 - a.dscaled;
+  const bool fast_ok = (kBM % G) == 0 && ((int64_t)G * a.total_q + stat_span) * 4 < (1ll << 32) && 32 * a.qs_tok_bytes < (1ll << 32);
   const int tok_per_blk = kBM / G;
   uint32_t voff_q[2], voff_s;
-  int tok_s;
+  int tok_l;  // token, within a block that starts at a token boundary, of row l32
   {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -168,50 +172,44 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       const int tq = div_group(rl);
       voff_q[i] = (uint32_t)(tq * a.qs_tok_bytes + (rl - tq * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(rl)) << 4));
     }
-    const int rs = wave * 8 + (lane & 7);
-    tok_s = div_group(rs);
-    voff_s = (uint32_t)((((int64_t)(rs - tok_s * G)) * a.total_q + tok_s) * 4);
+    tok_l = div_group(l32);
+    const int64_t which = (g == 0) == (a.lse2 < a.dscaled) ? 0 : stat_span;  // lanes < 32: lse2, the others: -delta
+    voff_s = (uint32_t)((((int64_t)(l32 - tok_l * G)) * a.total_q + tok_l + which) * 4);
   }
-  const float *stat_base = a.lse2 + (int64_t)kvh * G * a.total_q + q0;
-  const int64_t stat_delta = a.dscaled - a.lse2;
-  auto issue_tile = [&](int stage, int mbx) {
+  const uint8_t *q_task = reinterpret_cast<const uint8_t *>(a.q) + qbase;     // token 0 of the task, first head of the group
+  const uint8_t *do_task = reinterpret_cast<const uint8_t *>(a.dout) + qbase;
+  const float *stat_task = stat_lo + (int64_t)kvh * G * a.total_q + q0;
+  const uint32_t m0_wave = lds0 + wave * 8 * kRow;  // + stage * kTileBytes [+ kTileDO] [+ 4 * kRow]
+  auto block_is_fast = [&](int mbx) { return fast_ok && mbx >= bot && (mbx + 1) * kBM <= nrows; };
+  auto issue_fast = [&](int stage, int mbx) {
+    const int tok0 = mbx * tok_per_blk;
+    const uint32_t stat = kStatOff + stage * kStatBytes;
+    int lm = a.causal ? tok0 + tok_l + shift : lk - 1;
+    if (lm > lk - 1) lm = lk - 1;
+    reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[l32] = lm;
+    const int64_t tb = (int64_t)tok0 * a.qs_tok_bytes;
+    const uint32_t m0 = m0_wave + stage * kTileBytes;
+    lds_direct_load16(q_task + tb, voff_q[0], m0 + kTileQ);
+    lds_direct_load16(do_task + tb, voff_q[0], m0 + kTileDO);
+    lds_direct_load16(q_task + tb, voff_q[1], m0 + kTileQ + 4 * kRow);
+    lds_direct_load16(do_task + tb, voff_q[1], m0 + kTileDO + 4 * kRow);
+    lds_direct_load4_base(stat_task + tok0, voff_s, lds0 + stat);
+  };
+  auto issue_slow = [&](int stage, int mbx) {
     const int tile = stage * kTileBytes;
     const int stat = kStatOff + stage * kStatBytes;
     const bool blk_ok = mbx >= bot;
-    if (fast_ok && blk_ok && (mbx + 1) * kBM <= nrows) {
-      const int tok0 = mbx * tok_per_blk;
-      if (lane < 8) {
-        int lm = a.causal ? tok0 + tok_s + shift : lk - 1;
-        if (lm > lk - 1) lm = lk - 1;
-        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[wave * 8 + lane] = lm;
-        lds_direct_load4_base(stat_base + tok0, voff_s, lds0 + stat + wave * 32);
-        lds_direct_load4_base(stat_base + stat_delta + tok0, voff_s, lds0 + stat + kBM * 4 + wave * 32);
-      }
-      const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
-      const uint8_t *db = reinterpret_cast<const uint8_t *>(a.dout) + qbase + (int64_t)tok0 * a.qs_tok_bytes;
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const uint32_t dst = lds0 + tile + (wave * 8 + 4 * i) * kRow;
-        lds_direct_load16(qb, voff_q[i], dst + kTileQ);
-        lds_direct_load16(db, voff_q[i], dst + kTileDO);
-      }
-      return;
-    }
-    {  // row statistics: lanes 0..7 take one of the wave's eight rows each
-      const int rl = wave * 8 + (lane & 7);
-      const int rho = mbx * kBM + rl;
+    {  // row statistics and limits
+      const int rho = mbx * kBM + l32;
       const bool ok = blk_ok && rho < nrows;
       const int rc = ok ? rho : nrows - 1;
       const int tok = div_group(rc);
       const int hg = rc - tok * G;
-      if (lane < 8) {
-        int lm = a.causal ? tok + shift : lk - 1;
-        if (lm > lk - 1) lm = lk - 1;
-        reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[rl] = ok ? lm : -1;
-        const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
-        lds_direct_load4(a.lse2 + so, lds0 + stat + wave * 32);
-        lds_direct_load4(a.dscaled + so, lds0 + stat + kBM * 4 + wave * 32);
-      }
+      int lm = a.causal ? tok + shift : lk - 1;
+      if (lm > lk - 1) lm = lk - 1;
+      reinterpret_cast<int *>(lds + stat + 2 * kBM * 4)[l32] = ok ? lm : -1;
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok;
+      lds_direct_load4((g == 0 ? a.lse2 : a.dscaled) + so, lds0 + stat);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -228,6 +226,10 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       lds_direct_load16_ptr(qs + chunk * 8, dst + kTileQ);
       lds_direct_load16_ptr(ds + chunk * 8, dst + kTileDO);
     }
+  };
+  auto issue_tile = [&](int stage, int mbx) {
+    if (block_is_fast(mbx)) issue_fast(stage, mbx);
+    else issue_slow(stage, mbx);
   };
 
   const float c = a.scale * kLog2e;
