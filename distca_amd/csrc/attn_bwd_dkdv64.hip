@@ -3,7 +3,7 @@
 // One workgroup of 4 waves per (task, block of 256 keys, kv head), one wave per SIMD, so that a wave may use the
 // SIMD's whole register file: the dK^T / dV^T accumulators of its 64 keys (2 key blocks x 4 blocks over d x 2
 // matrices x 16 registers) fill the 256 accumulation registers, K of its keys stays in 64 vector registers as MFMA
-// B operand, V of the workgroup's keys in LDS.  The query side (Q, dO and the row statistics of every head of the
+// B operand, V of the workgroup's keys in LDS (and, as far as registers allow, in registers too: kVRegSlices).  The query side (Q, dO and the row statistics of every head of the
 // kv group, flattened into rows) streams through LDS in blocks of 32 rows, by LDS-direct loads into a ring of
 // four stages, from the last block down to the first one the causal mask lets see these keys.
 //
@@ -43,6 +43,10 @@ constexpr int kStatBytes = 3 * kBM * 4;  // lse2, -delta, lim per row
 constexpr int kStatOff = kStages * kTileBytes;
 constexpr int kVPitch = 272;             // resident V rows (padded: 128-bit row reads without bank conflicts)
 constexpr int kVOff = kStatOff + kStages * kStatBytes;
+// Of the eight 16-element slices over d of a wave's V rows, the first kVRegSlices stay in registers as B operands
+// beside K (as many as fit without spills inside the block loops: 12 fewer of a block's 72 LDS reads, -2 %); the
+// rest is read from LDS every block.
+constexpr int kVRegSlices = 6;
 constexpr int kLds = kVOff + kBN * kVPitch;
 static_assert(kLds <= 160 * 1024, "LDS budget");
 #ifndef DISTCA_RAWBAR
@@ -119,8 +123,8 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   auto div_group = [&](int n) { return a.group_magic ? (int)__umulhi((uint32_t)n, a.group_magic) : n; };
 
   // ---- K of the wave's keys as B operands (lane holds key 32 kb + l32, d = 16 s + 8 g .. +7); V of the same keys
-  // into LDS, read back by this wave only
-  elemx8 kreg[2][8];
+  // into LDS, read back by this wave only, and its first kVRegSlices slices into registers as well
+  elemx8 kreg[2][8], vreg[2][kVRegSlices];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int key = kw0 + 32 * kb + l32;
@@ -133,6 +137,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
         vf = *reinterpret_cast<const elemx8 *>(a.v + off + 16 * s);
       }
       kreg[kb][s] = kf;
+      if (s < kVRegSlices) vreg[kb][s] = vf;
       *reinterpret_cast<elemx8 *>(lds + kVOff + (wave * 64 + 32 * kb + l32) * kVPitch + 32 * s + 16 * g) = vf;
     }
   }
@@ -275,8 +280,10 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     auto load_q = [&](int s, int buf) { qa[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileQ + (a_rd ^ (s << 5))); };
     auto load_dv = [&](int s, int buf) {
       da[buf] = *reinterpret_cast<const elemx8 *>(tile + kTileDO + (a_rd ^ (s << 5)));
-      vb[buf][0] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * s);
-      vb[buf][1] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * kVPitch + 32 * s);
+      if (s >= kVRegSlices) {
+        vb[buf][0] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * s);
+        vb[buf][1] = *reinterpret_cast<const elemx8 *>(lds + v_rd + 32 * kVPitch + 32 * s);
+      }
     };
     load_q(0, 0);
     load_q(1, 1);
@@ -320,13 +327,13 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       fence();
-      mfma32_v(dpacc[0], da[s & 1], vb[s & 1][0]);
+      mfma32_v(dpacc[0], da[s & 1], s < kVRegSlices ? vreg[0][s < kVRegSlices ? s : 0] : vb[s & 1][0]);
       fence();
       p_elem(0, 2 * s);
       p_elem(0, 2 * s + 1);
       if (s == 4) p_cvt(0, 0);
       fence();
-      mfma32_v(dpacc[1], da[s & 1], vb[s & 1][1]);
+      mfma32_v(dpacc[1], da[s & 1], s < kVRegSlices ? vreg[1][s < kVRegSlices ? s : 0] : vb[s & 1][1]);
       fence();
       p_elem(1, 2 * s);
       p_elem(1, 2 * s + 1);
