@@ -5,7 +5,7 @@
 // matrices x 16 registers) fill the 256 accumulation registers, K of its keys stays in 64 vector registers as MFMA
 // B operand, V of the workgroup's keys in LDS (and, as far as registers allow, in registers too: kVRegSlices).  The query side (Q, dO and the row statistics of every head of the
 // kv group, flattened into rows) streams through LDS in blocks of 32 rows, by LDS-direct loads into a ring of
-// four stages, from the last block down to the first one the causal mask lets see these keys.
+// four stages, from the last block down to the first one the causal mask lets see these keys, or from that one up.
 //
 // With one wave per SIMD nothing else can use the SIMD's vector ALU while the wave waits for the matrix pipe, and
 // a wave issues in order: an MFMA that finds the pipe busy holds up everything behind it.  So the arithmetic of a
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   // or one piece of them (sched.h)
   int top = nmb, bot = mb0;
   {
-    const int piece = it4.w & 0xffff, pieces = it4.w >> 16;
+    const int piece = item_piece(it4.w), pieces = item_pieces(it4.w);
     if (pieces > 1) {
       const int n = nmb > mb0 ? nmb - mb0 : 0;
       top = nmb - piece_begin(n, piece, pieces);
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   const uint8_t *do_task = reinterpret_cast<const uint8_t *>(a.dout) + qbase;
   const float *stat_task = stat_lo + (int64_t)kvh * G * a.total_q + q0;
   const uint32_t m0_wave = lds0 + wave * 8 * kRow;  // + stage * kTileBytes [+ kTileDO] [+ 4 * kRow]
-  auto block_is_fast = [&](int mbx) { return fast_ok && mbx >= bot && (mbx + 1) * kBM <= nrows; };
+  auto block_is_fast = [&](int mbx) { return fast_ok && mbx >= bot && mbx < top && (mbx + 1) * kBM <= nrows; };
   auto issue_fast = [&](int stage, int mbx) {
     const int tok0 = mbx * tok_per_blk;
     const uint32_t stat = kStatOff + stage * kStatBytes;
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   auto issue_slow = [&](int stage, int mbx) {
     const int tile = stage * kTileBytes;
     const int stat = kStatOff + stage * kStatBytes;
-    const bool blk_ok = mbx >= bot;
+    const bool blk_ok = mbx >= bot && mbx < top;
     {  // row statistics and limits
       const int rho = mbx * kBM + l32;
       const bool ok = blk_ok && rho < nrows;
@@ -245,9 +245,13 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
   const int t_rd = (4 * g + i4) * kRow + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*(j&3) ^ 16*hi
 
   wait_vm<0>();  // K and V have arrived; the counted waits below cover the tile loads only
+  // The item's blocks are walked downwards from block top - 1 or upwards from block bot, as the schedule says
+  // (sched.h, kWalkUp: items of alternate rounds meet at the same query rows, which their XCD's L2 then serves).
+  const bool walk_up = (it4.w & kWalkUp) != 0;
+  auto block_at = [&](int p) { return walk_up ? bot + p : top - 1 - p; };
   if (niter > 0) {
-    issue_tile(0, top - 1);
-    issue_tile(1, top - 2);
+    issue_tile(0, block_at(0));
+    issue_tile(1, block_at(1));
   }
 
   // One block.  MASKED: the block straddles the diagonal or the end of the task, compare and select per element.
@@ -387,10 +391,10 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     }
   };
 
-  // Blocks are visited from the last one down, so the furthest key a block's rows see only falls from block to
-  // block: first come blocks that see all of this wave's keys from every row (no masking), then blocks on the
-  // diagonal (masked), then, for waves whose keys lie past the diagonal of the remaining blocks, blocks that see
-  // none of them.  Each kind has a loop of its own with one body (with the two bodies and a skip in one loop the
+  // Along a walk the furthest key a block's rows see only falls (downwards) or only grows (upwards) from block to
+  // block: blocks that see all of this wave's keys from every row (no masking), blocks on the diagonal (masked)
+  // and, for waves whose keys lie past the diagonal of some blocks, blocks that see none of them come in that
+  // order or in the reverse.  Each kind has a loop of its own with one body (with the two bodies and a skip in one loop the
   // register allocator moved the 256 accumulators between the register files in every iteration); every wave
   // passes the same barriers and makes the same requests in all of them.  A block cut off by the end of the task
   // needs no masking on that account: its missing rows are zero rows of Q and dO, which add nothing to dK or dV
@@ -413,20 +417,29 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
     __syncthreads();
 #endif
     // stage (p + 2) % 4 was last read for block p - 2, which every wave left before this barrier
-    issue_tile((p + 2) % kStages, top - 1 - (p + 2));
+    issue_tile((p + 2) % kStages, block_at(p + 2));
   };
+  // 2: every row of the block sees all of this wave's keys; 1: some rows see some; 0: none does
+  auto block_kind = [&](int p) {
+    const int mbx = block_at(p);
+    if (kw0 + 63 <= row_limit(mbx * kBM)) return 2;
+    int rho_last = (mbx + 1) * kBM - 1;
+    if (rho_last > nrows - 1) rho_last = nrows - 1;
+    return kw0 <= row_limit(rho_last) ? 1 : 0;
+  };
+  // Along a walk the kinds come in the order 2, 1, 0 (downwards) or 0, 1, 2 (upwards): five loops in a row, of
+  // which a walk uses three.
   int p = 0;
-  for (; p < niter; ++p) {
-    const int mbx = top - 1 - p;
-    if (kw0 + 63 > row_limit(mbx * kBM)) break;  // the block's first row does not see all of the wave's keys
+  for (; p < niter && block_kind(p) == 0; ++p) advance(p);
+  for (; p < niter && block_kind(p) == 1; ++p) {
+    advance(p);
+    block(p % kStages, std::true_type{});
+  }
+  for (; p < niter && block_kind(p) == 2; ++p) {
     advance(p);
     block(p % kStages, std::false_type{});
   }
-  for (; p < niter; ++p) {
-    const int mbx = top - 1 - p;
-    int rho_last = (mbx + 1) * kBM - 1;
-    if (rho_last > nrows - 1) rho_last = nrows - 1;
-    if (kw0 > row_limit(rho_last)) break;  // no row of this block, or of any below it, sees a key of this wave
+  for (; p < niter && block_kind(p) == 1; ++p) {
     advance(p);
     block(p % kStages, std::true_type{});
   }

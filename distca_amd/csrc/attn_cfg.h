@@ -52,6 +52,7 @@ inline int validate_params(const distca_ca_params *p) {
 inline SchedGeom fwd_geom(const distca_ca_params *p) {
   SchedGeom g;
   g.split_target = 0;
+  g.walk_round = 0;
   g.rows_per_block = kFwdRows;
   g.kv_per_block = kFwdKV;
   g.group = p->num_heads_q / p->num_heads_kv;
@@ -92,6 +93,8 @@ inline SchedGeom bwd_geom(const distca_ca_params *p) {
   g.causal = p->causal != 0;
   g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_q * g.group / kBwdRows + 1);
   g.split_target = bwd_split_target(p);
+  // one round of the dK/dV list per kv head: as many items as compute units serve that head (sched.h, kWalkUp)
+  g.walk_round = num_compute_units() / p->num_heads_kv > 0 ? num_compute_units() / p->num_heads_kv : 1;
   return g;
 }
 // Upper bound of the item count that needs only host-known sizes.

@@ -136,6 +136,27 @@ __global__ __launch_bounds__(kSchedThreads) void build_schedule_kernel(const int
     }
   }
   __syncthreads();
+  // 5. (backward) walk direction by rank.  The scatter above puts the entries of one cost bin in whatever order
+  // the threads came; an entry's rank in the order (bin, task, block, piece) is the start of its bin plus the
+  // number of entries of the bin that precede it in that order, counted here, and is the same in every run.
+  if (BWD && g.walk_round > 0) {
+    const int32_t total = bins[0] < max_items ? bins[0] : max_items;
+    for (int32_t pos = tid; pos < total; pos += kSchedThreads) {
+      const int4 it = reinterpret_cast<const int4 *>(items)[pos];
+      const int32_t bin = cost_bin(g, it.z);
+      const int32_t seg0 = bin == kSchedBins - 1 ? 0 : bins[bin + 1];  // bins lie from the most expensive down
+      const int32_t seg1 = bins[bin] < total ? bins[bin] : total;
+      const int64_t key = ((int64_t)(base[it.x] + it.y) << 16) | item_piece(it.w);
+      int32_t rank = seg0;
+      for (int32_t o = seg0; o < seg1 && seg1 - seg0 <= kWalkTieLimit; ++o) {
+        const int4 ot = reinterpret_cast<const int4 *>(items)[o];
+        rank += (((int64_t)(base[ot.x] + ot.y) << 16) | item_piece(ot.w)) < key;
+      }
+      // only the flag bit changes, and the reads above look at the other bits only
+      if ((rank / g.walk_round) & 1) items[4 * pos + 3] = it.w | kWalkUp;
+    }
+    __syncthreads();
+  }
   if (tid == 0) {
     // after the scatter the counter of the cheapest bin holds the number of entries
     const int32_t total = bins[0];
@@ -219,6 +240,12 @@ extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const 
   }
   std::stable_sort(v.begin(), v.end(), [](const It &a, const It &b) { return a.bin > b.bin; });
   const int64_t n = (int64_t)v.size();
+  if (kind == 1 && g.walk_round > 0)
+    for (int64_t s0 = 0, s1; s0 < n; s0 = s1) {  // one cost bin: entries [s0, s1)
+      for (s1 = s0 + 1; s1 < n && v[s1].bin == v[s0].bin; ++s1) {}
+      for (int64_t e = s0; e < s1; ++e)
+        if (((s1 - s0 <= kWalkTieLimit ? e : s0) / g.walk_round) & 1) v[e].piece |= kWalkUp;
+    }
   for (int64_t e = 0; e < n && e < max_items; ++e) {
     items[4 * e + 0] = v[e].task;
     items[4 * e + 1] = v[e].block;

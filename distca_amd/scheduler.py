@@ -56,7 +56,8 @@ def build_schedule(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequenc
                    num_heads_kv: int, head_dim: int = 128, causal: bool = True, deterministic: bool = False,
                    total_k: int | None = None) -> np.ndarray:
     """Work items as an int32 array [n, 4] of (task, block, cost, piece | pieces << 16), most expensive
-    first.  Backward items of a batch too small to occupy the device are cut into pieces of
+    first; in a backward list bit 31 of the fourth word (WALK_UP) marks items walked upwards from the diagonal
+    (`item_piece`, `item_pieces` take the word apart).  Backward items of a batch too small to occupy the device are cut into pieces of
     consecutive query blocks unless `deterministic`; everything else has pieces = 1, piece = 0."""
     cu_q = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
     cu_k = np.ascontiguousarray(cu_seqlens_k, dtype=np.int32)
@@ -72,6 +73,17 @@ def build_schedule(kind: int, cu_seqlens_q: Sequence[int], cu_seqlens_k: Sequenc
         m = lib.distca_ca_schedule_host(kind, cu_q.ctypes.data, cu_k.ctypes.data, ctypes.byref(p), items.ctypes.data, int(n))
         assert m == n
     return items
+
+
+WALK_UP = -(1 << 31)   # bit 31 of an item's fourth word, as int32
+
+
+def item_piece(w):
+    return w & 0xffff
+
+
+def item_pieces(w):
+    return (w >> 16) & 0x7fff
 
 
 def whole_items(items: np.ndarray) -> np.ndarray:

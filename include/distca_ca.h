@@ -255,7 +255,12 @@ int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off,
  * the device and p->deterministic is 0, a key block is cut into pieces of
  * consecutive query blocks, whose dK/dV the kernel adds up in fp32).  Writes
  * up to max_items (task, block, cost, piece | pieces << 16) quadruples sorted
- * by descending cost and returns the item count, or a negative error.  The reference has no counterpart: flash-attn launches a static
+ * by descending cost and returns the item count, or a negative error.  In a
+ * backward list bit 31 of the fourth word marks the items whose query blocks
+ * the kernel walks upwards from the diagonal instead of downwards from the
+ * end (alternate rounds of as many items as compute units serve a kv head, so
+ * that items running side by side stream the same rows): piece = word &
+ * 0xffff, pieces = (word >> 16) & 0x7fff.  The reference has no counterpart: flash-attn launches a static
  * (m-block, batch, head) grid sized by max_seqlen_q.
  * ------------------------------------------------------------------------- */
 int64_t distca_ca_schedule_host(int kind, const int32_t *cu_seqlens_q,

@@ -136,6 +136,30 @@ def test_single_documents_around_the_piece_cutting_threshold(cuda, hq, hkv, n):
     assert_close_bf16(dv, ref_dv, "dv", **tol)
 
 
+def test_key_blocks_walked_in_both_directions(cuda):
+    """The dK/dV list marks alternate rounds of items (as many as compute units serve a kv head: 16 here) to be
+    walked upwards from the diagonal instead of downwards from the end.  Whole key blocks (deterministic), prefix
+    tasks among them: both directions occur, the gradients match the oracle and a second run bit for bit."""
+    from distca_amd import scheduler
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    q_lens, k_lens, hq, hkv = [2600, 900, 1800, 37], [2600, 2100, 1800, 300], 16, 16
+    items = scheduler.build_schedule(scheduler.BWD, cu(q_lens), cu(k_lens), hq, hkv, deterministic=True)
+    up = items[:, 3] < 0
+    assert up.any() and (~up).any() and (scheduler.item_pieces(items[:, 3]) == 1).all()
+    cu_q, cu_k = cu(q_lens), cu(k_lens)
+    q, k, v, do = make_qkv(int(cu_q[-1]), int(cu_k[-1]), hq, hkv, 128, 77)
+    dq_, dk_ = torch.tensor(cu_q, device=cuda), torch.tensor(cu_k, device=cuda)
+    qd, kd, vd, dod = q.to(cuda), k.to(cuda), v.to(cuda), do.to(cuda)
+    out, lse = ca_varlen_fwd(qd, kd, vd, dq_, dk_, max(q_lens), max(k_lens))
+    a = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dq_, dk_, max(q_lens), max(k_lens), None, True, True, None)
+    b = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dq_, dk_, max(q_lens), max(k_lens), None, True, True, None)
+    torch.cuda.synchronize()
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    ref = ca_reference_bwd(do, q, k, v, cu_q, cu_k, out=out.cpu(), softmax_lse=lse.cpu())
+    for x, r, name in zip(a, ref, ("dq", "dk", "dv")):
+        assert_close_bf16(x, r, name)
+
+
 def test_empty_task(cuda):
     _run([128, 0, 70], [128, 0, 70], 4, 2, 8, cuda)
 
