@@ -10,7 +10,13 @@ namespace distca {
 
 struct BwdArgs {
   const elem_t *q, *k, *v, *dout;
-  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and -delta
+  const float *lse2, *dscaled;  // [Hq][Tq]: lse*log2e and -delta, written by the dQ kernel, read by the dK/dV kernel
+  // what the dQ kernel makes them from: O laid out like q and dout, and the forward's lse either as [Hq][Tq] or as Hq
+  // floats per token in the query-side region (first byte of that part in token 0), one of the two null
+  const elem_t *out;
+  const float *lse;
+  const uint8_t *lse_tok;
+  float *lse2_w, *dscaled_w;
   elem_t *dq, *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;

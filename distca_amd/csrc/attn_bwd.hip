@@ -9,16 +9,17 @@
 // dQ partial sums with fp32 atomics was measured first: the atomics alone (4 bytes per
 // (row, key) pair per 128 keys, 124 GB at 128K tokens) took as long as the rest of the kernel.
 //
-//   1. bwd_prepare_kernel: per (token, head) row, scale*<dO, O> and lse*log2(e) -> workspace.
-//   2. ca_bwd_dkdv64_kernel (attn_bwd_dkdv64.hip): dK and dV, one workgroup of 4 waves per (task, block of
-//      256 keys, kv head), in the order of the backward tile schedule.
-//   3. ca_bwd_dq_kernel: one workgroup of 8 waves per (task, block of 256 flattened query
+//   1. ca_bwd_dq_kernel: one workgroup of 8 waves per (task, block of 256 flattened query
 //      rows, kv head), in the order of the forward tile schedule; the mirror image of the
 //      forward kernel.  Q and dO stay in registers as B operands, K/V tiles of 64 keys are
 //      streamed through LDS:
 //        S^T = K Q^T, dP^T = V dO^T        A from LDS rows, B from registers
 //        P, dS as above (one query row per lane: lse2 and delta are per-lane scalars)
 //        dQ^T += K^T dS^T                  A by transposing LDS reads of the K tile, B = dS registers
+//      Its prologue, which reads a row's dO anyway, also makes the row statistics both kernels need
+//      (delta = <dO, O>, lse * log2(e)) and leaves them in the workspace.
+//   2. ca_bwd_dkdv64_kernel (attn_bwd_dkdv64.hip): dK and dV, one workgroup of 4 waves per (task, block of
+//      256 keys, kv head), in the order of the backward tile schedule.
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 #include "api_util.h"
@@ -88,19 +89,33 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
     const int64_t ro = qs_task + (int64_t)tok[m] * a.qs_tok_bytes + ((kvh * G + hg) * kHeadDim + 8 * g) * 2;  // bytes
     lse2[m] = INFINITY;  // rows past the task: P = exp2(-inf) = 0
     dsc[m] = 0.f;
-    if (valid[m]) {
-      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
-      lse2[m] = a.lse2[so];
-      dsc[m] = -a.dscaled[so] * a.scale;
-    }
+    // The row statistics of the backward are made here, where the row's dO is read anyway, and left in the
+    // workspace for the dK/dV kernel, which runs after this one: delta = <dO, O> over the row (this lane's half of
+    // d, then the sum of the lane pair) and lse in the log2 domain.
+    float part = 0.f;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       if (valid[m]) {
         qf[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s);
         dof[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
+        const elemx8 of = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.out) + ro + 32 * s);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)of[i];
       } else {
         qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
         dof[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    const float delta = pair_sum(part);
+    if (valid[m]) {
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
+      const float l = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
+                                : a.lse[so];
+      lse2[m] = l * kLog2e;
+      dsc[m] = delta * a.scale;
+      if (g == 0) {
+        a.lse2_w[so] = lse2[m];
+        a.dscaled_w[so] = -delta;  // the start value of the dP accumulators in the dK/dV kernel
       }
     }
   }
@@ -304,58 +319,6 @@ __global__ __launch_bounds__(kWaves * 64, (MSUB == 1 && kWaves == 4 ? 2 : 1)) vo
   }
 }
 
-// Per (token, head) row: dscaled[h][t] = -sum_d dO*O (minus delta, unscaled; the name is historical) and lse2[h][t] = lse[h][t]*log2(e).
-// dout and out point at their part of token 0 of a region laid out like BwdArgs' query side; lse is
-// [Hq][Tq] fp32, or, when lse_tok is given instead, Hq fp32 per token at lse_tok + token start.
-__global__ __launch_bounds__(256) void bwd_prepare_kernel(const uint8_t *__restrict__ dout, const uint8_t *__restrict__ out,
-                                                         const float *__restrict__ lse, const uint8_t *__restrict__ lse_tok,
-                                                         const int64_t *__restrict__ task_off, int64_t tok_bytes,
-                                                         const int32_t *__restrict__ cu_q, int32_t num_tasks,
-                                                         float *__restrict__ dscaled, float *__restrict__ lse2, int64_t rows,
-                                                         int32_t hq, int32_t total_q, float scale) {
-  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int sub = threadIdx.x & 15;
-  float s = 0.f;
-  int64_t t = 0, tok_start = 0;
-  int h = 0;
-  bool live = row < rows;
-  if (live) {
-    t = row / hq;
-    h = (int)(row - t * hq);
-    // tokens past the last task (total_q may exceed the tasks' rows) belong to no shard: nothing is read for them,
-    // and their statistics make P = exp2(s - inf) = 0 wherever a kernel might look
-    live = t < cu_q[num_tasks];
-  }
-  if (live) {
-    if (task_off) {
-      // the task that holds token t: last b with cu_q[b] <= t
-      int lo = 0, hi = num_tasks - 1;
-      while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (cu_q[mid] <= t) lo = mid;
-        else hi = mid - 1;
-      }
-      tok_start = task_off[lo] + (t - cu_q[lo]) * tok_bytes;
-    } else {
-      tok_start = t * tok_bytes;
-    }
-    const int64_t eo = tok_start + (int64_t)h * (kHeadDim * 2) + sub * 16;
-    const elemx8 a = *reinterpret_cast<const elemx8 *>(dout + eo);
-    const elemx8 b = *reinterpret_cast<const elemx8 *>(out + eo);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s += (float)a[i] * (float)b[i];
-  }
-#pragma unroll
-  for (int o = 8; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
-  if (row < rows && sub == 0) {
-    const int64_t o = (int64_t)h * total_q + t;
-    dscaled[o] = -s;  // minus delta, unscaled: the start value of the dP accumulators in dkdv
-    float l = INFINITY;
-    if (live) l = lse_tok ? reinterpret_cast<const float *>(lse_tok + tok_start)[h] : lse[o];
-    lse2[o] = l * kLog2e;
-  }
-}
-
 // Zeroes the dk / dv rows that no workgroup of the dK/dV kernel writes when every task owns its K/V rows: the
 // rows of tasks without queries (they get no work item) and the rows past the last task.  Workgroup (b, y):
 // part y of task b's rows, b == num_tasks standing for the tail.
@@ -513,14 +476,11 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   }
   if (p->num_tasks == 0 || p->total_q == 0) return check_launch("ca_bwd(clear)");
 
-  const int64_t rows = (int64_t)p->total_q * p->num_heads_q;
-  hipLaunchKernelGGL(bwd_prepare_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, s, (const uint8_t *)dout,
-                     (const uint8_t *)out, qs.lse, (const uint8_t *)qs.lse_tok, qs.task_off, qs.tok_bytes, cu_q, p->num_tasks,
-                     (float *)(ws + w.delta), (float *)(ws + w.lse2), rows, p->num_heads_q, p->total_q, p->softmax_scale);
-
   BwdArgs a;
   a.q = (const elem_t *)q; a.k = (const elem_t *)k; a.v = (const elem_t *)v; a.dout = (const elem_t *)dout;
   a.lse2 = (const float *)(ws + w.lse2); a.dscaled = (const float *)(ws + w.delta);
+  a.lse2_w = (float *)(ws + w.lse2); a.dscaled_w = (float *)(ws + w.delta);
+  a.out = (const elem_t *)out; a.lse = qs.lse; a.lse_tok = (const uint8_t *)qs.lse_tok;
   a.dq = (elem_t *)dq; a.dk = (elem_t *)dk; a.dv = (elem_t *)dv;
   a.qs_task_off = qs.task_off; a.qs_tok_bytes = qs.tok_bytes; a.dq_task_off = qs.dq_task_off; a.dq_tok_bytes = qs.dq_tok_bytes;
   a.dk_acc = use_acc ? (float *)(ws + w.dk_acc) : nullptr;
@@ -539,6 +499,21 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     device_setup_done(kSlotBwdLds);
   }
 
+  // ---- dQ: one workgroup per (task, block of query rows, kv head).  It runs first: it also leaves the row
+  // statistics (lse in the log2 domain, -delta) in the workspace, which the dK/dV kernel reads.
+  {
+    const SchedGeom geom = dq_geom(p);
+    const int64_t max_items = dq_max_items(p);
+    rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
+    if (rc) return rc;
+    const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
+    if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
+    a.sched = (const int32_t *)(ws + w.sched_q);
+    a.zero_row = ws + w.sched_q + sched_zero_row_off(p->num_tasks, max_items);
+    a.tickets = (int32_t *)(ws + w.sched_q + sched_ticket_off(p->num_tasks, max_items));
+    ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
+    hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
+  }
   // ---- dK, dV: one workgroup per (task, 256-key block, kv head)
   {
     const SchedGeom geom = bwd_geom(p);
@@ -556,20 +531,6 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, s);
     if (rc) return rc;
-  }
-  // ---- dQ: one workgroup per (task, block of query rows, kv head)
-  {
-    const SchedGeom geom = dq_geom(p);
-    const int64_t max_items = dq_max_items(p);
-    rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
-    if (rc) return rc;
-    const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
-    if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
-    a.sched = (const int32_t *)(ws + w.sched_q);
-    a.zero_row = ws + w.sched_q + sched_zero_row_off(p->num_tasks, max_items);
-    a.tickets = (int32_t *)(ws + w.sched_q + sched_ticket_off(p->num_tasks, max_items));
-    ScopedTimer timer(DISTCA_TIMER_CA_BWD_DQ, s);
-    hipLaunchKernelGGL((ca_bwd_dq_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kWaves * 64), kDqLds, s, a);
   }
   if (use_acc) {
     hipLaunchKernelGGL(cvt_elem_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (const float *)(ws + w.dk_acc), (elem_t *)dk, kv_elems / 8);
