@@ -246,6 +246,38 @@ def test_prefix_tasks_equal_whole_document(cuda):
     assert_close_bf16(dv_s, dv_w.float(), "dv", max_abs=3e-2)
 
 
+def test_device_walk_marks_equal_host_mirror_with_many_equal_documents(cuda):
+    """A hundred documents of one length: every cost bin of the dK/dV list holds a hundred entries, more than the
+    builder ranks against each other, so all entries of a bin take the mark of its first one; a second batch of
+    distinct lengths, where every entry is ranked.  The device list carries the marks of the host mirror, entry by
+    entry (as sets: entries of one bin may come in any order), and is the same in a second run."""
+    from distca_amd import scheduler, workloads
+    from distca_amd._lib import CaParams, load
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    import ctypes
+    hq, hkv = 8, 8
+    for lens in ([1536] * 100, list(range(300, 300 + 37 * 60, 37))):
+        ql = np.asarray(lens, dtype=np.int64)
+        b = workloads.TaskBatch("walk_marks", ql, ql, hq, hkv)
+        q, k, v, do, cu_q, cu_k = _dev_inputs(b, hq, hkv, cuda, 5)
+        mq = int(ql.max())
+        p = CaParams(len(ql), b.total_q, b.kv_rows, hq, hkv, 128, mq, mq, 128 ** -0.5, 1, 1, 0)
+        nbytes = load().distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+        host = scheduler.build_schedule(scheduler.BWD, b.cu_seqlens_q, b.cu_seqlens_k, hq, hkv, deterministic=True)
+        assert (host[:, 3] < 0).any() and (host[:, 3] > 0).any()
+        header = (4 + len(ql) + 1 + 3) // 4 * 4
+        lists = []
+        for run in range(2):
+            ws = torch.zeros((nbytes,), dtype=torch.uint8, device=cuda)
+            out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mq)
+            ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mq, None, True, True, None, workspace=ws)
+            torch.cuda.synchronize()
+            w = ws.cpu().view(torch.int32).numpy()
+            assert int(w[0]) == len(host) and int(w[2]) == 0
+            lists.append(sorted(map(tuple, w[header:header + 4 * len(host)].reshape(-1, 4).tolist())))
+        assert lists[0] == lists[1] == sorted(map(tuple, host.tolist()))
+
+
 @pytest.mark.parametrize("kind", ["fwd", "bwd"])
 def test_device_schedule_equals_host_mirror(cuda, kind):
     """The workspace begins with the schedule the device built ([0] = item count, then the

@@ -199,3 +199,14 @@ def test_walk_flags_alternate_by_rounds_of_the_list(hq, hkv):
     assert (scheduler.item_pieces(items[:, 3]) == 1).all() and (scheduler.item_piece(items[:, 3]) == 0).all()
     fwd = scheduler.build_schedule(scheduler.FWD, _cu(lq), _cu(lk), hq, hkv)
     assert (fwd[:, 3] == 1 << 16).all()
+
+
+def test_walk_flags_of_a_bin_too_large_to_rank():
+    """Entries of one cost bin are ranked among themselves only up to 64 of them; a hundred documents of one length
+    put a hundred entries into every bin, and all of them take the mark that the bin's first entry would get."""
+    items = scheduler.build_schedule(scheduler.BWD, _cu([1536] * 100), _cu([1536] * 100), 8, 8, deterministic=True)
+    costs, up = items[:, 2], items[:, 3] < 0
+    rnd = 256 // 8
+    for c in np.unique(costs):
+        idx = np.flatnonzero(costs == c)
+        assert len(idx) == 100 and (up[idx] == bool((idx[0] // rnd) & 1)).all()
