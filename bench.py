@@ -241,6 +241,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--no-pack", action="store_true")
     ap.add_argument("--no-tick", action="store_true")
+    ap.add_argument("--no-probe", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the CA-server path; --gpus must be 1 "
@@ -304,6 +305,27 @@ def main():
     log(f"  ca_fwd_kernel {fwd_k:.3f} ms -> {fwd_tf:.1f} TFLOP/s ({100 * fwd_tf / PEAK_BF16_TFLOPS:.1f}%)")
     log(f"  ca_bwd kernels {bwd_k:.3f} ms (dkdv {dkdv_k:.3f} + dq {dq_k:.3f}) -> {bwd_tf:.1f} TFLOP/s ({100 * bwd_tf / PEAK_BF16_TFLOPS:.1f}%)")
 
+    # what this device delivers for the MFMA instruction itself, right after the attention steps (the part is warm):
+    # a loop of MFMAs on every SIMD, alone and with other work in every MFMA's shadow
+    probe = None
+    if not args.no_probe:
+        scratch = torch.zeros(4, dtype=torch.int64, device=dev)
+        stream_ptr = torch.cuda.current_stream().cuda_stream
+        probe = {}
+        for name, kind in (("mfma_only", _lib.PROBE_MFMA_ONLY), ("with_1kb_lds_read_per_mfma", _lib.PROBE_LDS_READ),
+                           ("with_4_fma_per_mfma", _lib.PROBE_FMA4), ("with_2_exp_per_mfma", _lib.PROBE_EXP2)):
+            for _ in range(3):  # the last of three runs: the clock has settled by then
+                tf, cyc, ghz = _lib.probe_mfma_rate(kind, 20000, scratch.data_ptr(), stream_ptr)
+            probe[name] = {"TFLOP/s": round(tf, 1), "cycles_per_mfma": round(cyc, 2), "clock_GHz": round(ghz, 3)}
+        executed = 1e-12 * (flop_fwd + 1.4 * flop_bwd) / ((fwd_k + bwd_k) * 1e-3)  # S and dP are computed in both backward kernels
+        probe["executed_TFLOP/s_of_the_three_attention_kernels"] = round(executed, 1)
+        probe["executed_over_mfma_only"] = round(executed / probe["mfma_only"]["TFLOP/s"], 4)
+        probe["note"] = ("v_mfma_f32_32x32x16_bf16 on pseudo-random operands, one wave per SIMD on every SIMD, 160000 per wave; "
+                         "rate by HIP events, clock by the device's cycle and real-time counters: what the power limit leaves "
+                         "of the published 2.5 PFLOP/s (every pipe busy at 2.4 GHz) on this device for this instruction")
+        log(f"  MFMA-only loop {probe['mfma_only']['TFLOP/s']} TFLOP/s at {probe['mfma_only']['clock_GHz']} GHz; the attention kernels execute "
+            f"{probe['executed_TFLOP/s_of_the_three_attention_kernels']} TFLOP/s = {100 * probe['executed_over_mfma_only']:.1f} % of it")
+
     pack = None
     if not args.no_pack:
         del dq, dk, dv
@@ -341,6 +363,7 @@ def main():
                      "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv64_kernel": round(dkdv_k, 4), "ca_bwd_dq_kernel": round(dq_k, 4)},
                      "executed_tflops": {"ca_bwd_dkdv64_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
                      "launches": bwd_n,
+                     "mfma_probe": probe,
                      "also": {"ca_fwd_kernel": {"achieved": round(fwd_tf, 2), "frac": round(fwd_tf / PEAK_BF16_TFLOPS, 4),
                                                 "avg_launch_ms": round(fwd_k, 4), "launches": fwd_n}}},
         "cpu_baseline": cpu,

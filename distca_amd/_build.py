@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libdistca_ca.so")
-SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]
+SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip", "probe.hip"]
 # The attention kernels exist once per element type: the same sources compiled again with -DDISTCA_F16 give the fp16
 # kernels and their launchers under names of their own; the entry points (compiled once) pick by distca_ca_params.dtype.
 F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]

@@ -62,6 +62,8 @@ SYMBOLS = {
     "distca_timing_enable": (None, [c_int]),
     "distca_timing_read": (c_int, [c_int, POINTER(ctypes.c_double), POINTER(c_int64)]),
     "distca_ca_tile_shape": (c_int, [c_int, POINTER(CaParams), POINTER(c_int32 * 2)]),
+    "distca_probe_mfma_rate": (c_int, [c_int, c_int, c_void_p, POINTER(ctypes.c_double), POINTER(ctypes.c_double),
+                                       POINTER(ctypes.c_double), c_void_p]),
 }
 
 _lib = None
@@ -99,6 +101,19 @@ def timing_read(which: int):
     ms, n = ctypes.c_double(0), c_int64(0)
     check(load().distca_timing_read(which, ctypes.byref(ms), ctypes.byref(n)), "timing_read")
     return ms.value, n.value
+
+
+PROBE_MFMA_ONLY, PROBE_LDS_READ, PROBE_FMA4, PROBE_EXP2 = range(4)
+
+
+def probe_mfma_rate(kind: int, iters: int, scratch_ptr: int, stream_ptr: int = 0):
+    """(TFLOP/s, cycles per MFMA, shader clock in GHz) of a loop of MFMAs on every SIMD of the device, with
+    nothing (PROBE_MFMA_ONLY), an LDS read, four FMAs or two exponentials behind every MFMA.  `scratch_ptr`: 32
+    bytes of device memory.  Synchronises the stream."""
+    tf, cyc, ghz = ctypes.c_double(0), ctypes.c_double(0), ctypes.c_double(0)
+    check(load().distca_probe_mfma_rate(kind, iters, scratch_ptr, ctypes.byref(tf), ctypes.byref(cyc), ctypes.byref(ghz),
+                                        stream_ptr), "probe_mfma_rate")
+    return tf.value, cyc.value, ghz.value
 
 
 def check(rc: int, what: str) -> None:

@@ -296,6 +296,23 @@ int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
 void distca_timing_enable(int on);
 int distca_timing_read(int which, double *total_ms, int64_t *launches);
 
+/* ---------------------------------------------------------------------------
+ * What the device delivers for the MFMA instruction the attention kernels are
+ * made of, measured on the spot.  No counterpart in the reference: a
+ * diagnostic for benchmarks, which print it beside the kernels' own rate.  One
+ * wave on every SIMD issues 8 * iters v_mfma_f32_32x32x16_bf16 on pseudo-random
+ * operands and, behind every MFMA, nothing (kind 0), one 1 KB LDS read (1),
+ * four v_fma_f32 (2) or two v_exp_f32 (3): work that fits into the MFMA's
+ * shadow, so that the pipe stays fully occupied and the result shows what the
+ * power limit leaves of the clock.  Returns the MFMA rate in TFLOP/s (by HIP
+ * events on `stream`), the cycles per MFMA and the shader clock in GHz (by the
+ * device's cycle and real-time counters).  scratch32: 32 bytes of device
+ * memory.  Synchronises `stream`.
+ * ------------------------------------------------------------------------- */
+int distca_probe_mfma_rate(int kind, int iters, void *scratch32, double *tflops,
+                           double *cycles_per_mfma, double *clock_ghz,
+                           void *stream);
+
 #ifdef __cplusplus
 }
 #endif

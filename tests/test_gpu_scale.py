@@ -469,3 +469,19 @@ def test_server_ticks_in_place_equal_step_by_step_at_full_size(cuda):
         sends.append(send)
     torch.cuda.synchronize()
     assert torch.equal(sends[0], sends[1])
+
+
+def test_mfma_rate_probe(cuda):
+    """The diagnostic loop of MFMAs: the pipe is fully occupied (33 cycles per MFMA, also with an LDS read, four FMAs
+    or two exponentials in every MFMA's shadow), the clock is a plausible one, and the rate is what they imply."""
+    from distca_amd import _lib
+    scratch = torch.zeros(4, dtype=torch.int64, device=cuda)
+    for kind in (_lib.PROBE_MFMA_ONLY, _lib.PROBE_LDS_READ, _lib.PROBE_FMA4, _lib.PROBE_EXP2):
+        tf, cyc, ghz = _lib.probe_mfma_rate(kind, 20000, scratch.data_ptr())
+        print(f"probe kind {kind}: {tf:.0f} TFLOP/s, {cyc:.1f} cycles per MFMA, {ghz:.2f} GHz", flush=True)
+        assert 31.5 <= cyc <= 37.0 and 0.8 <= ghz <= 2.6
+        n_simd = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+        by_counters = 32768 * n_simd * ghz / cyc / 1e3   # of the one wave that reads them; the slowest XCD sets the events' time
+        assert 0.8 * by_counters <= tf <= 1.03 * by_counters
+    with pytest.raises(RuntimeError):
+        _lib.probe_mfma_rate(9, 10, scratch.data_ptr())
