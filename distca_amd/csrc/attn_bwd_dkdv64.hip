@@ -74,6 +74,9 @@ __device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
 __device__ __forceinline__ void mfma32_v0(f32x16 &acc, elemx8 a, elemx8 b) {  // acc = A B
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
 }
+__device__ __forceinline__ void mfma32_vc(f32x16 &acc, elemx8 a, elemx8 b, const f32x16 &c0) {  // acc = A B + c0
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "v"(b), "v"(c0));
+}
 
 template <bool ALIAS>
 __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
@@ -270,14 +273,13 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
       lse_buf[cq & 1] = *reinterpret_cast<const f32x4 *>(stat + qr * 4);
       if constexpr (kMasked) lim_buf[cq & 1] = *reinterpret_cast<const i32x4 *>(stat + 2 * kBM * 4 + qr * 4);
     };
+    // -delta of the rows, loaded into the registers of the first key half's dP accumulator, is also the C operand of
+    // the first dP MFMA of the second key half, which is issued first (no copy)
 #pragma unroll
     for (int cq = 0; cq < 4; ++cq) {
       const f32x4 nd = *reinterpret_cast<const f32x4 *>(stat + kBM * 4 + (8 * cq + 4 * g) * 4);
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        dpacc[0][4 * cq + rr] = nd[rr];
-        dpacc[1][4 * cq + rr] = nd[rr];
-      }
+      for (int rr = 0; rr < 4; ++rr) dpacc[0][4 * cq + rr] = nd[rr];
     }
     // ---- step 1: S = Q K^T
     elemx8 qa[2], da[2], vb[2][2];
@@ -331,13 +333,18 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dkdv64_kernel(BwdArgs a) {
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       fence();
-      mfma32_v(dpacc[0], da[s & 1], s < kVRegSlices ? vreg[0][s < kVRegSlices ? s : 0] : vb[s & 1][0]);
+      if (s == 0) {
+        mfma32_vc(dpacc[1], da[0], vreg[1][0], dpacc[0]);
+        mfma32_v(dpacc[0], da[0], vreg[0][0]);
+      } else {
+        mfma32_v(dpacc[0], da[s & 1], s < kVRegSlices ? vreg[0][s < kVRegSlices ? s : 0] : vb[s & 1][0]);
+      }
       fence();
       p_elem(0, 2 * s);
       p_elem(0, 2 * s + 1);
       if (s == 4) p_cvt(0, 0);
       fence();
-      mfma32_v(dpacc[1], da[s & 1], s < kVRegSlices ? vreg[1][s < kVRegSlices ? s : 0] : vb[s & 1][1]);
+      if (s > 0) mfma32_v(dpacc[1], da[s & 1], s < kVRegSlices ? vreg[1][s < kVRegSlices ? s : 0] : vb[s & 1][1]);
       fence();
       p_elem(1, 2 * s);
       p_elem(1, 2 * s + 1);
