@@ -10,7 +10,7 @@ to stderr.
 
 Algorithmic work: causal pairs P = sum_tasks [Lq*Lk - Lq(Lq-1)/2]; forward 4*Hq*D*P FLOP,
 backward 10*Hq*D*P FLOP.  `roofline` describes the dominant kernels, the two that make up the
-attention backward (ca_bwd_dkdv64_kernel over key blocks, ca_bwd_dq_kernel over query blocks):
+attention backward (ca_bwd_dkdv64_kernel over key blocks, ca_bwd_dq64_kernel over query blocks):
 algorithmic backward FLOPs over the sum of their launch durations, measured live by HIP events
 the library records on the launch stream.  Both recompute S and dP, so together they execute
 14*Hq*D*P FLOP for 10*Hq*D*P of algorithmic work; `executed_tflops` reports that rate per kernel.
@@ -35,7 +35,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
 # WRITE_SIZE (x1.000), factors from the pack kernels' known copy sizes in the same run
-MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.94e9, "ca_bwd_dkdv64_kernel": 23.76e9, "ca_bwd_dq_kernel": 17.10e9}
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.94e9, "ca_bwd_dkdv64_kernel": 23.76e9, "ca_bwd_dq64_kernel": 17.10e9}
 
 
 def log(*a):
@@ -356,12 +356,12 @@ def main():
                                f"{tq} packed tokens, 32q/8kv heads, d=128, causal, fwd+bwd",
                    "causal_pairs": batch.causal_pairs, "flop_fwd": flop_fwd, "flop_bwd": flop_bwd,
                    "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2)},
-        "roofline": {"bound": "mfma", "kernel": "ca_bwd_dkdv64_kernel + ca_bwd_dq_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "ca_bwd_dkdv64_kernel + ca_bwd_dq64_kernel", "achieved": round(bwd_tf, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(bwd_tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": (MEASURED_TRAFFIC_BYTES["ca_bwd_dkdv64_kernel"] + MEASURED_TRAFFIC_BYTES["ca_bwd_dq_kernel"]) if default_workload else None,
+                     "traffic": (MEASURED_TRAFFIC_BYTES["ca_bwd_dkdv64_kernel"] + MEASURED_TRAFFIC_BYTES["ca_bwd_dq64_kernel"]) if default_workload else None,
                      "traffic_unit": "bytes per launch (both kernels)",
-                     "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv64_kernel": round(dkdv_k, 4), "ca_bwd_dq_kernel": round(dq_k, 4)},
-                     "executed_tflops": {"ca_bwd_dkdv64_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
+                     "avg_launch_ms": round(bwd_k, 4), "avg_launch_ms_parts": {"ca_bwd_dkdv64_kernel": round(dkdv_k, 4), "ca_bwd_dq64_kernel": round(dq_k, 4)},
+                     "executed_tflops": {"ca_bwd_dkdv64_kernel": round(0.8 * flop_bwd / dkdv_k / 1e9, 1), "ca_bwd_dq64_kernel": round(0.6 * flop_bwd / dq_k / 1e9, 1)},
                      "launches": bwd_n,
                      "mfma_probe": probe,
                      "also": {"ca_fwd_kernel": {"achieved": round(fwd_tf, 2), "frac": round(fwd_tf / PEAK_BF16_TFLOPS, 4),

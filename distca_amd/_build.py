@@ -14,10 +14,10 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libdistca_ca.so")
-SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip", "probe.hip"]
+SOURCES = ["api.cpp", "pack.hip", "sched.hip", "attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip", "attn_bwd_dq64.hip", "probe.hip"]
 # The attention kernels exist once per element type: the same sources compiled again with -DDISTCA_F16 give the fp16
 # kernels and their launchers under names of their own; the entry points (compiled once) pick by distca_ca_params.dtype.
-F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip"]
+F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_bwd_dkdv64.hip", "attn_bwd_dq64.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-x", "hip",
@@ -42,7 +42,7 @@ def _hipcc() -> str:
 # Flags a source must not be compiled with.  attn_bwd_dkdv64.hip wants the compiler's default MFMA form (results in
 # the accumulation registers) for its 256 dK/dV accumulators; the accumulators its vector ALU touches are pinned
 # to vector registers in the source.
-DROP_FLAGS = {"attn_bwd_dkdv64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+DROP_FLAGS = {"attn_bwd_dkdv64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "attn_bwd_dq64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 
 def _compile(src: str, obj: str, extra: list[str]) -> None:

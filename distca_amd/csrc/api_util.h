@@ -48,9 +48,9 @@ void device_setup_done(int slot);
 // Every kernel that needs such set-up exists once per element type; the fp16 builds of the sources use the upper half.
 enum { kSlotPerType = 3, kSlotCount = 2 * kSlotPerType };
 #ifdef DISTCA_F16
-enum { kSlotFwdLds = kSlotPerType + 0, kSlotBwdLds = kSlotPerType + 1, kSlotBwdLds64 = kSlotPerType + 2 };
+enum { kSlotFwdLds = kSlotPerType + 0, kSlotBwdDq64 = kSlotPerType + 1, kSlotBwdLds64 = kSlotPerType + 2 };
 #else
-enum { kSlotFwdLds = 0, kSlotBwdLds = 1, kSlotBwdLds64 = 2 };
+enum { kSlotFwdLds = 0, kSlotBwdDq64 = 1, kSlotBwdLds64 = 2 };
 #endif
 
 }  // namespace distca

@@ -64,5 +64,8 @@ int run_fwd_tokens_f16(const void *q_base, const int64_t *q_task_off, int64_t q_
 int dkdv64_lds_bytes();
 int launch_dkdv64(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);       // bf16 elements
 int launch_dkdv64_f16(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);   // fp16 elements
+// The dQ kernel with 64 query rows per wave (attn_bwd_dq64.hip).
+int launch_dq64(const BwdArgs &a, int64_t grid, hipStream_t stream);
+int launch_dq64_f16(const BwdArgs &a, int64_t grid, hipStream_t stream);
 
 }  // namespace distca

@@ -1,0 +1,415 @@
+// dQ of the varlen causal attention backward for gfx950, 64 query rows per wave.
+//
+// One workgroup of 4 waves per (task, block of 256 flattened query rows, kv head), one wave per SIMD with the
+// SIMD's whole register file.  A wave owns two sub-blocks of 32 rows: their Q and dO stay in registers as MFMA B
+// operands, their dQ^T accumulators in the accumulation registers.  K/V tiles of 32 keys stream through a ring of
+// four LDS stages by LDS-direct loads, from key 0 up to the last key the block's rows see; every LDS fragment a
+// wave reads (K rows, V rows, transposed K) feeds two MFMAs, one per sub-block: half the LDS bytes per MFMA of
+// a wave that owns 32 rows.  With one wave per SIMD the arithmetic of a tile is written between the MFMAs of the
+// same tile, as in the dK/dV kernel (attn_bwd_dkdv64.hip):
+//
+//   step 1   S^T  = K Q^T        16 MFMAs   A: rows of the K tile (LDS), B: Q registers
+//   step 2   dP^T = V dO^T       16 MFMAs   A: rows of the V tile, B: dO registers      beside them: P from S
+//   step 3   dQ^T += K^T dS^T    16 MFMAs   A: transposing reads of the K tile, B: dS   of the tile before; beside
+//                                           them: dS = P (dP - delta) of this tile
+//
+// The prologue also makes the row statistics of the backward (delta = <dO, O>, lse in the log2 domain) and leaves
+// them in the workspace for the dK/dV kernel, which runs after this one.
+#include "api_util.h"
+#include "attn_bwd.h"
+#include "attn_cfg.h"
+#include "common.h"
+
+#include <type_traits>
+
+namespace distca {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRowsWg = 256;            // flattened query rows per workgroup (kDqRows)
+constexpr int kKeys = 32;               // keys per tile
+constexpr int kRow = 256;               // bytes per tile row, chunks swizzled by tile_swz
+constexpr int kTile = kKeys * kRow;
+constexpr int kStageBytes = 2 * kTile;  // K tile, V tile
+constexpr int kStages = 4;
+constexpr int kLds = kStages * kStageBytes;
+constexpr int kLoadsPerTile = 4;        // vector-memory instructions a wave issues per tile
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kLead = 2;                // fragments by which sub-block 0 leads in the dQ step
+constexpr int kFrags = 4;               // transposed K fragments held at a time
+static_assert(kDqRows == kRowsWg, "the dQ work list is built for blocks of 256 rows");
+
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void fence() { __builtin_amdgcn_sched_barrier(0); }
+// The S and dP accumulators are read and overwritten by the vector ALU and must live in vector registers; this file
+// is compiled with the compiler's default MFMA form (results in the accumulation registers, right for dQ), so
+// these MFMAs are written as assembly.  The compiler does not space such an instruction from the vector
+// instructions that read its result: the order below keeps a later MFMA, or enough other instructions, between.
+__device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_v0(f32x16 &acc, elemx8 a, elemx8 b) {  // acc = A B
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_vc(f32x16 &acc, elemx8 a, elemx8 b, const f32x16 &c0) {  // acc = A B + c0
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "v"(b), "v"(c0));
+}
+// The same with the B operand in accumulation registers, where Q lives: a wave's 512 registers are 256 of each
+// kind, and the vector half is what the tile arithmetic is short of.
+typedef float accop_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ accop_t to_acc_regs(elemx8 v) {
+  accop_t r;
+  asm volatile("; operand to accumulation registers" : "=a"(r) : "0"(__builtin_bit_cast(accop_t, v)));
+  return r;
+}
+__device__ __forceinline__ void mfma32_va(f32x16 &acc, elemx8 a, accop_t b) {
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma32_va0(f32x16 &acc, elemx8 a, accop_t b) {
+  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+}
+
+__global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int nitems = a.sched[0];
+  int item, kvh;
+  if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
+  const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  const int task = it4.x, mblk = it4.y;
+
+  const int q0 = a.cu_q[task];
+  const int64_t qs_task = a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes;
+  const int64_t dq_task = a.dq_task_off ? a.dq_task_off[task] : (int64_t)q0 * a.dq_tok_bytes;
+  const int lq = a.cu_q[task + 1] - q0;
+  const int lk = a.cu_k[task + 1] - a.cu_k[task];
+  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
+  const int G = a.group;
+  const int shift = lk - lq;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int row_wg = mblk * kRowsWg;
+  const int nrows = lq * G;
+
+  int tok_end = (row_wg + kRowsWg + G - 1) / G;
+  if (tok_end > lq) tok_end = lq;
+  int nvis = a.causal ? tok_end + shift : lk;
+  if (nvis > lk) nvis = lk;
+  const int ntiles = nvis > 0 ? (nvis + kKeys - 1) / kKeys : 0;
+
+  // ---- this lane's two rows: Q and dO as B operands (row l32 of a sub-block, d = 16 s + 8 g .. +7), statistics
+  int row[2], tok[2], lim[2];
+  bool valid[2];
+  float lse2[2], delta[2];
+  accop_t qf[2][8];
+  elemx8 dof[2][8];
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    row[m] = row_wg + (wave * 2 + m) * 32 + l32;
+    valid[m] = row[m] < nrows;
+    tok[m] = row[m] / G;
+    const int hg = row[m] - tok[m] * G;
+    int lm = a.causal ? tok[m] + shift : lk - 1;
+    if (lm > lk - 1) lm = lk - 1;
+    lim[m] = lm;
+    const int64_t ro = qs_task + (int64_t)tok[m] * a.qs_tok_bytes + ((kvh * G + hg) * kHeadDim + 8 * g) * 2;  // bytes
+    lse2[m] = INFINITY;  // rows past the task: P = exp2(-inf) = 0
+    float part = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      if (valid[m]) {
+        qf[m][s] = to_acc_regs(*reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s));
+        dof[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
+        const elemx8 of = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.out) + ro + 32 * s);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)of[i];
+      } else {
+        qf[m][s] = to_acc_regs(elemx8{0, 0, 0, 0, 0, 0, 0, 0});
+        dof[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    delta[m] = pair_sum(part);  // this lane's half of d, then the sum of the lane pair
+    if (valid[m]) {
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
+      const float l = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
+                                : a.lse[so];
+      lse2[m] = l * kLog2e;
+      if (g == 0) {
+        a.lse2_w[so] = lse2[m];
+        a.dscaled_w[so] = -delta[m];  // the start value of the dP accumulators in the dK/dV kernel
+      }
+    }
+  }
+  // -delta of the lane's row in all 16 registers of a vector: the C operand of a tile's first dP MFMA, so that
+  // dS = P * (what the MFMAs leave) costs one instruction per element
+  f32x16 ndl[2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ndl[m][r] = -delta[m];
+  const int wrow0 = row_wg + wave * 64;
+  int wrow1 = wrow0 + 63;
+  if (wrow1 > nrows - 1) wrow1 = nrows - 1;
+  const bool wave_live = wrow0 < nrows;
+  int lim_first = 0x7fffffff, lim_last = -1;
+  if (wave_live) {
+    lim_first = a.causal ? wrow0 / G + shift : lk - 1;
+    if (lim_first > lk - 1) lim_first = lk - 1;
+    lim_last = a.causal ? wrow1 / G + shift : lk - 1;
+    if (lim_last > lk - 1) lim_last = lk - 1;
+  }
+
+  // ---- K/V tile fetch: this wave brings rows 8 w .. 8 w + 7 of the K tile and of the V tile, four rows per
+  // instruction.  Tiles that lie wholly inside the prefix take a form without per-lane address arithmetic (a scalar
+  // base that advances by one tile, per-lane offsets that never change); rows past the prefix read the zero row.
+  const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
+  const elem_t *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  uint32_t voff[2];
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii) {
+    const int r = 8 * wave + 4 * ii + (lane >> 4);
+    voff[ii] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
+  }
+  auto issue_tile = [&](int stage, int j) {
+    const uint32_t dst = lds0 + stage * kStageBytes + 8 * wave * kRow;
+    if ((j + 1) * kKeys <= lk) {
+      const elem_t *kt = kbase + (int64_t)j * kKeys * kv_stride, *vt = vbase + (int64_t)j * kKeys * kv_stride;
+      lds_direct_load16(kt, voff[0], dst);
+      lds_direct_load16(kt, voff[1], dst + 4 * kRow);
+      lds_direct_load16(vt, voff[0], dst + kTile);
+      lds_direct_load16(vt, voff[1], dst + kTile + 4 * kRow);
+      return;
+    }
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const int r = 8 * wave + 4 * ii + (lane >> 4);
+      const int key = j * kKeys + r;
+      const int chunk = (lane & 15) ^ tile_swz(r);
+      const bool ok = key < lk;
+      const elem_t *kp = ok ? kbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
+      const elem_t *vp = ok ? vbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
+      lds_direct_load16_ptr(kp + chunk * 8, dst + 4 * ii * kRow);
+      lds_direct_load16_ptr(vp + chunk * 8, dst + kTile + 4 * ii * kRow);
+    }
+  };
+
+  f32x16 dqacc[2][4];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dqacc[m][db][r] = 0.f;
+  const float c = a.scale * kLog2e;
+  const int k_rd = l32 * kRow + ((g ^ tile_swz(l32)) << 4);  // A operand rows of a tile, ^ 32*s
+  // transposed K operand: lane points at (key 4g + i4 [+8 hi +16 t], chunk 8 b4 + h1 [+2 db], half lane&1);
+  // tile_swz of that row is (i4<<1) | (g<<3) | hi
+  const int i4 = (lane & 15) >> 2, b4 = (lane >> 4) & 1, h1 = (lane & 3) >> 1;
+  const int t_rd = (4 * g + i4) * kRow + ((((b4 ^ g) << 3) | (i4 << 1) | h1) << 4) + 8 * (lane & 1);  // ^ 32*db ^ 16*hi
+
+  // Absolute LDS addresses of this lane's operand reads in stage 0, the eight swizzled variants of each read shape,
+  // kept in registers: where the stage is a constant (the unrolled loop below) stage and tile sit in the read
+  // instruction's offset field and no address arithmetic is left between the MFMAs.
+  uint32_t k_ad[8], t_ad[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    k_ad[i] = lds0 + (k_rd ^ (i << 5));
+    t_ad[i] = lds0 + ((t_rd ^ ((i & 3) << 5) ^ ((i >> 2) << 4)) + (i >> 2) * 8 * kRow);
+    asm volatile("" : "+v"(k_ad[i]), "+v"(t_ad[i]));
+  }
+
+  wait_vm<0>();  // Q, dO, O have arrived; the counted waits below cover the tile loads only
+  if (ntiles > 0) {
+    issue_tile(0, 0);
+    issue_tile(1, 1);
+  }
+
+  // One tile.  MASKED: the tile straddles the diagonal or the end of the prefix, compare and select per element.
+  auto tile = [&](auto stage, int key0, auto masked) __attribute__((always_inline)) {  // stage: an int or a constant
+    constexpr bool kMasked = decltype(masked)::value;
+    const uint32_t so = (uint32_t)stage * kStageBytes;
+    f32x16 sacc[2], dpacc[2];
+    elemx8 kf[2], vf[2];
+    elemx4 ct[kFrags][2];
+    auto load_k = [&](int s, int buf) { kf[buf] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(k_ad[s] + so)); };
+    auto load_v = [&](int s, int buf) { vf[buf] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(k_ad[s] + so + kTile)); };
+    auto load_t = [&](int n, int buf) {  // n = 4 t + db: keys 16 t .. 16 t + 15, d block db
+      ct[buf][0] = lds_read_tr(lds_ptr(t_ad[n & 3] + so + 16 * (n >> 2) * kRow));
+      ct[buf][1] = lds_read_tr(lds_ptr(t_ad[4 + (n & 3)] + so + 16 * (n >> 2) * kRow));
+    };
+    // ---- step 1: S^T = K Q^T
+    load_k(0, 0);
+    load_k(1, 1);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      fence();
+      if (s == 0) {
+        mfma32_va0(sacc[0], kf[0], qf[0][0]);
+        mfma32_va0(sacc[1], kf[0], qf[1][0]);
+      } else {
+        mfma32_va(sacc[0], kf[s & 1], qf[0][s]);
+        mfma32_va(sacc[1], kf[s & 1], qf[1][s]);
+      }
+      fence();
+      if (s + 2 < 8) load_k(s + 2, s & 1);
+      if (s >= 6) load_v(s - 6, s - 6);  // the first operands of step 2
+    }
+    // ---- step 2: dP^T = V dO^T; beside the MFMAs, P = exp2(S c - lse2) of two elements per MFMA
+    auto p_elem = [&](int m, int r) {
+      float p = fast_exp2(__builtin_fmaf(sacc[m][r], c, -lse2[m]));
+      if constexpr (kMasked) {
+        if (key0 + acc_row(r, g) > lim[m]) p = 0.f;
+      }
+      sacc[m][r] = p;
+    };
+    auto ds_elem = [&](int m, int r) { dpacc[m][r] = sacc[m][r] * dpacc[m][r]; };  // dP accumulated on top of -delta
+    elemx8 dsf[2][2];
+    auto ds_cvt = [&](int m, int t) {
+      const int r0 = 8 * t;
+      dsf[m][t] = cvt8(dpacc[m][r0], dpacc[m][r0 + 1], dpacc[m][r0 + 2], dpacc[m][r0 + 3], dpacc[m][r0 + 4], dpacc[m][r0 + 5],
+                       dpacc[m][r0 + 6], dpacc[m][r0 + 7]);
+    };
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      fence();
+      if (s == 0) mfma32_vc(dpacc[0], vf[0], dof[0][0], ndl[0]);
+      else mfma32_v(dpacc[0], vf[s & 1], dof[0][s]);
+      fence();
+      p_elem(0, 2 * s);
+      p_elem(0, 2 * s + 1);
+      fence();
+      if (s == 0) mfma32_vc(dpacc[1], vf[0], dof[1][0], ndl[1]);
+      else mfma32_v(dpacc[1], vf[s & 1], dof[1][s]);
+      fence();
+      p_elem(1, 2 * s);
+      p_elem(1, 2 * s + 1);
+      if (s + 2 < 8) load_v(s + 2, s & 1);
+      if (s >= 8 - kFrags) load_t(s - (8 - kFrags), s - (8 - kFrags));  // the first operands of step 3
+    }
+    fence();
+    // dS of the first 16 keys of sub-block 0: dP is complete only now
+#pragma unroll
+    for (int r = 0; r < 8; ++r) ds_elem(0, r);
+    ds_cvt(0, 0);
+    // ---- step 3: dQ^T += K^T dS^T.  Sub-block 0 leads by kLead fragments: dS of sub-block 1's first 16 keys stands
+    // behind its first MFMAs, dS of the other 16 keys of both behind the MFMAs that follow
+    static_assert(kLead == 2 && kFrags == 4, "the portions below are laid out for a lead of two fragments");
+#pragma unroll
+    for (int n = 0; n < kLead; ++n) {
+      const elemx8 kt = cat4(ct[n % kFrags][0], ct[n % kFrags][1]);
+      fence();
+      dqacc[0][n & 3] = mfma32(kt, dsf[0][0], dqacc[0][n & 3]);
+      fence();
+#pragma unroll
+      for (int r = 4 * n; r < 4 * n + 4; ++r) ds_elem(1, r);
+    }
+    ds_cvt(1, 0);
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+      const elemx8 kt1 = cat4(ct[n % kFrags][0], ct[n % kFrags][1]);
+      fence();
+      dqacc[1][n & 3] = mfma32(kt1, dsf[1][n >> 2], dqacc[1][n & 3]);
+      fence();
+      if (n + kFrags < 8) load_t(n + kFrags, n % kFrags);
+      if (n == 0) {
+#pragma unroll
+        for (int r = 8; r < 12; ++r) ds_elem(0, r);
+      }
+      if (n == 1) {
+#pragma unroll
+        for (int r = 12; r < 16; ++r) ds_elem(0, r);
+        ds_cvt(0, 1);
+      }
+      if (n == 2) {
+#pragma unroll
+        for (int r = 8; r < 12; ++r) ds_elem(1, r);
+      }
+      if (n == 3) {
+#pragma unroll
+        for (int r = 12; r < 16; ++r) ds_elem(1, r);
+        ds_cvt(1, 1);
+      }
+      if (n + kLead < 8) {
+        const int n0 = n + kLead;
+        const elemx8 kt0 = cat4(ct[n0 % kFrags][0], ct[n0 % kFrags][1]);
+        fence();
+        dqacc[0][n0 & 3] = mfma32(kt0, dsf[0][n0 >> 2], dqacc[0][n0 & 3]);
+        fence();
+      }
+    }
+  };
+
+  // Tiles are walked from key 0 up, so the first key of a tile only grows: first come tiles that every row of the
+  // wave sees whole (no masking), then tiles on the diagonal or at the end of the prefix (masked), then, for waves
+  // whose rows end below those of the block's last wave, tiles that none of their rows sees.  Each kind has a loop
+  // of its own with one body; every wave passes the same barriers and makes the same requests in all of them.
+  auto advance = [&](int p) {
+    wait_vm<kLoadsPerTile>();
+    fence();
+    asm volatile("s_barrier" ::: "memory");
+    fence();
+    issue_tile((p + 2) % kStages, p + 2);
+  };
+  int p = 0;
+  // four unmasked tiles per round, one per ring stage, as long as the fourth is still unmasked
+  for (; p + 3 < ntiles; p += 4) {
+    if (!wave_live || (p + 3) * kKeys + kKeys - 1 > lim_first) break;
+    advance(p);
+    tile(std::integral_constant<int, 0>{}, p * kKeys, std::false_type{});
+    advance(p + 1);
+    tile(std::integral_constant<int, 1>{}, (p + 1) * kKeys, std::false_type{});
+    advance(p + 2);
+    tile(std::integral_constant<int, 2>{}, (p + 2) * kKeys, std::false_type{});
+    advance(p + 3);
+    tile(std::integral_constant<int, 3>{}, (p + 3) * kKeys, std::false_type{});
+  }
+  for (; p < ntiles; ++p) {
+    if (!wave_live || p * kKeys + kKeys - 1 > lim_first) break;
+    advance(p);
+    tile(p % kStages, p * kKeys, std::false_type{});
+  }
+  for (; p < ntiles; ++p) {
+    if (!wave_live || p * kKeys > lim_last) break;
+    advance(p);
+    tile(p % kStages, p * kKeys, std::true_type{});
+  }
+  for (; p < ntiles; ++p) advance(p);
+  wait_vm<0>();  // nothing may still be on its way into LDS when the workgroup ends
+
+  // ---- epilogue: dQ rows (registers 4*cq..+3 of block db hold d0..d0+3)
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    if (valid[m]) {
+      const int hg = row[m] - tok[m] * G;
+      elem_t *op = reinterpret_cast<elem_t *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int cq = 0; cq < 4; ++cq) {
+          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
+          *reinterpret_cast<elemx4 *>(op + d0) = cvt4(dqacc[m][db][4 * cq] * a.scale, dqacc[m][db][4 * cq + 1] * a.scale,
+                                                      dqacc[m][db][4 * cq + 2] * a.scale, dqacc[m][db][4 * cq + 3] * a.scale);
+        }
+    }
+  }
+}
+
+}  // namespace
+
+int DISTCA_FN(launch_dq64)(const BwdArgs &a, int64_t grid, hipStream_t stream) {
+  if (device_setup_pending(kSlotBwdDq64)) {
+    hipError_t e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS: %s", kLds, hipGetErrorString(e));
+    device_setup_done(kSlotBwdDq64);
+  }
+  hipLaunchKernelGGL(ca_bwd_dq64_kernel, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
+  return DISTCA_OK;
+}
+
+}  // namespace distca

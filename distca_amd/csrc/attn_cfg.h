@@ -9,10 +9,6 @@
 namespace distca {
 
 constexpr int kHeadDim = 128;
-#ifndef DISTCA_DQ_WAVES
-#define DISTCA_DQ_WAVES 8
-#endif
-constexpr int kWaves = DISTCA_DQ_WAVES;  // waves per workgroup of the dQ kernel
 
 // Forward and dQ kernels: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles
 // of 64 keys.  One sub-tile keeps a wave under 256 registers, so a compute unit holds eight waves.
@@ -25,7 +21,7 @@ constexpr int kWaves = DISTCA_DQ_WAVES;  // waves per workgroup of the dQ kernel
 constexpr int kFwdMsub = DISTCA_FWD_MSUB;
 constexpr int kFwdWaves = DISTCA_FWD_WAVES;  // waves per workgroup of the forward kernel
 constexpr int kFwdRows = kFwdWaves * 32 * kFwdMsub;
-constexpr int kDqRows = kWaves * 32 * kFwdMsub;
+constexpr int kDqRows = 256;  // the dQ kernel: four waves of two 32-row sub-blocks
 constexpr int kFwdKV = 64;
 
 // Backward: a workgroup owns 256 keys (eight waves of 32, in two groups that work through the same

@@ -291,7 +291,7 @@ int distca_ca_tile_shape(int kind, const distca_ca_params *p, int32_t out[2]);
 #define DISTCA_TIMER_MEMCPY_NON_CP 2
 #define DISTCA_TIMER_MEMCPY_CP 3
 #define DISTCA_TIMER_GRAD_SUM 4
-#define DISTCA_TIMER_CA_BWD_DQ 5   /* ca_bwd_dq_kernel                       */
+#define DISTCA_TIMER_CA_BWD_DQ 5   /* ca_bwd_dq64_kernel                     */
 #define DISTCA_TIMER_COUNT 6
 void distca_timing_enable(int on);
 int distca_timing_read(int which, double *total_ms, int64_t *launches);
