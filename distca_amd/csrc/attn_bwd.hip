@@ -27,8 +27,6 @@
 namespace distca {
 namespace {
 
-constexpr float kLog2e = 1.4426950408889634f;
-
 // Zeroes the dk / dv rows that no workgroup of the dK/dV kernel writes when every task owns its K/V rows: the
 // rows of tasks without queries (they get no work item) and the rows past the last task.  Workgroup (b, y):
 // part y of task b's rows, b == num_tasks standing for the tail.

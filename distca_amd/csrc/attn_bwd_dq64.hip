@@ -10,8 +10,8 @@
 //
 //   step 1   S^T  = K Q^T        16 MFMAs   A: rows of the K tile (LDS), B: Q registers
 //   step 2   dP^T = V dO^T       16 MFMAs   A: rows of the V tile, B: dO registers      beside them: P from S
-//   step 3   dQ^T += K^T dS^T    16 MFMAs   A: transposing reads of the K tile, B: dS   of the tile before; beside
-//                                           them: dS = P (dP - delta) of this tile
+//   step 3   dQ^T += K^T dS^T    16 MFMAs   A: transposing reads of the K tile, B: dS   beside them: dS = P (dP - delta)
+//                                           of the keys and sub-block whose MFMAs come later in the step
 //
 // The prologue also makes the row statistics of the backward (delta = <dO, O>, lse in the log2 domain) and leaves
 // them in the workspace for the dK/dV kernel, which runs after this one.
@@ -50,9 +50,6 @@ __device__ __forceinline__ void fence() { __builtin_amdgcn_sched_barrier(0); }
 // instructions that read its result: the order below keeps a later MFMA, or enough other instructions, between.
 __device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma32_v0(f32x16 &acc, elemx8 a, elemx8 b) {  // acc = A B
-  asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void mfma32_vc(f32x16 &acc, elemx8 a, elemx8 b, const f32x16 &c0) {  // acc = A B + c0
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "v"(b), "v"(c0));
