@@ -74,6 +74,18 @@ def test_prefix_tasks_lk_gt_lq(cuda):
     _run([128, 200, 64], [384, 200, 1000], 8, 2, 4, cuda)
 
 
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4), (16, 2)])
+def test_prefix_lengths_around_tile_and_ring_boundaries(cuda, hq, hkv):
+    """Tasks whose K/V prefixes end one key before, on and one key after multiples of 32 (a K/V tile of the dQ
+    kernel), of 64 (a tile of the forward) and of 128 (one round of the dQ kernel's four ring stages), with query
+    shards of 1 to 100 tokens: workgroups with one to a dozen tiles, with and without unmasked tiles, whose last
+    waves own no row or only a few."""
+    k_lens = [1, 31, 32, 33, 63, 64, 65, 95, 97, 127, 128, 129, 159, 161, 191, 193, 255, 256, 257, 289, 383, 385]
+    q_lens = [1, 31, 17, 33, 5, 64, 65, 16, 97, 100, 3, 1, 64, 33, 100, 17, 8, 100, 65, 1, 100, 49]
+    assert all(q <= k for q, k in zip(q_lens, k_lens))
+    _run(q_lens, k_lens, hq, hkv, 21, cuda)
+
+
 def test_shared_kv_prefix(cuda):
     """Three shards of one 600-token document reading one stored KV copy."""
     _run([200, 150, 250], [200, 350, 600], 8, 2, 5, cuda, kv_offsets=[0, 0, 0], total_k=600)
