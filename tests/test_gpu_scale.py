@@ -477,11 +477,13 @@ def test_mfma_rate_probe(cuda):
     from distca_amd import _lib
     scratch = torch.zeros(4, dtype=torch.int64, device=cuda)
     for kind in (_lib.PROBE_MFMA_ONLY, _lib.PROBE_LDS_READ, _lib.PROBE_FMA4, _lib.PROBE_EXP2):
-        tf, cyc, ghz = _lib.probe_mfma_rate(kind, 20000, scratch.data_ptr())
+        _lib.probe_mfma_rate(kind, 2000, scratch.data_ptr())   # the first launch of a kernel also loads it
+        tf, cyc, ghz = _lib.probe_mfma_rate(kind, 40000, scratch.data_ptr())
         print(f"probe kind {kind}: {tf:.0f} TFLOP/s, {cyc:.1f} cycles per MFMA, {ghz:.2f} GHz", flush=True)
         assert 31.5 <= cyc <= 37.0 and 0.8 <= ghz <= 2.6
         n_simd = 4 * torch.cuda.get_device_properties(0).multi_processor_count
-        by_counters = 32768 * n_simd * ghz / cyc / 1e3   # of the one wave that reads them; the slowest XCD sets the events' time
-        assert 0.8 * by_counters <= tf <= 1.03 * by_counters
+        # the counters are those of one wave; the events also see the launch, and the slowest XCD sets their time
+        by_counters = 32768 * n_simd * ghz / cyc / 1e3
+        assert 0.6 * by_counters <= tf <= 1.05 * by_counters
     with pytest.raises(RuntimeError):
         _lib.probe_mfma_rate(9, 10, scratch.data_ptr())
