@@ -20,6 +20,8 @@ struct BwdArgs {
   elem_t *dq, *dk, *dv;
   float *dk_acc, *dv_acc;  // used instead of dk/dv when tasks may alias KV rows
   const int32_t *cu_q, *cu_k, *kv_off;
+  // the dK/dV list over groups of tasks that share stored K/V rows (sched.h, SharedGroups); null otherwise
+  const int32_t *grp_first, *grp_tasks, *grp_off, *grp_lmax;
   const int32_t *sched;
   int32_t *tickets;  // one counter per kv head (sched.h)
   const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
@@ -62,8 +64,9 @@ int run_fwd_tokens_f16(const void *q_base, const int64_t *q_task_off, int64_t q_
 
 // The dK/dV kernel with 64 keys per wave (attn_bwd_dkdv64.hip): LDS bytes it needs, and its launch.
 int dkdv64_lds_bytes();
-int launch_dkdv64(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);       // bf16 elements
-int launch_dkdv64_f16(const BwdArgs &a, int64_t grid, bool alias, hipStream_t stream);   // fp16 elements
+// atomic_sums: items add to the fp32 accumulators (pieces of key blocks); shared: items are (group of tasks, key block)
+int launch_dkdv64(const BwdArgs &a, int64_t grid, bool atomic_sums, bool shared, hipStream_t stream);       // bf16 elements
+int launch_dkdv64_f16(const BwdArgs &a, int64_t grid, bool atomic_sums, bool shared, hipStream_t stream);   // fp16 elements
 // The dQ kernel with 64 query rows per wave (attn_bwd_dq64.hip).
 int launch_dq64(const BwdArgs &a, int64_t grid, hipStream_t stream);
 int launch_dq64_f16(const BwdArgs &a, int64_t grid, hipStream_t stream);

@@ -6,8 +6,9 @@
 // The backward runs as two kernels that both recompute P from (Q, K, LSE), so that neither
 // needs floating-point atomics and the result is bit-reproducible (the `deterministic` switch
 // of the reference's FlashAttnArgs holds by construction).  A single-kernel form that added
-// dQ partial sums with fp32 atomics was measured first: the atomics alone (4 bytes per
-// (row, key) pair per 128 keys, 124 GB at 128K tokens) took as long as the rest of the kernel.
+// dQ partial sums with fp32 atomics was measured first: the atomics alone (a 16 KB patch per
+// 32 rows x 256 keys, 62 GB at 131 072 tokens, at the 1.3 TB/s the device adds floats at) took
+// longer than the two kernels together.
 //
 //   1. ca_bwd_dq64_kernel (attn_bwd_dq64.hip): dQ, one workgroup of 4 waves per (task, block of 256 flattened
 //      query rows, kv head), in the order of the forward tile schedule.  Its prologue, which reads a row's dO
@@ -52,6 +53,21 @@ __global__ __launch_bounds__(256) void fill_unowned_rows_kernel(u32x4 *__restric
   }
 }
 
+// The same for tasks over shared stored rows: zeroes the stored rows no group of tasks covers (sched.h, SharedGroups:
+// gap u, u <= num_tasks; those past the number of groups are empty).  Workgroup (u, y): part y of gap u.
+__global__ __launch_bounds__(256) void fill_gap_rows_kernel(u32x4 *__restrict__ dk, u32x4 *__restrict__ dv,
+                                                           const int32_t *__restrict__ gap_lo, const int32_t *__restrict__ gap_hi,
+                                                           int32_t total_k, int64_t row_vecs) {
+  int64_t r0 = gap_lo[blockIdx.x], r1 = gap_hi[blockIdx.x];
+  if (r0 < 0) r0 = 0;
+  if (r1 > total_k) r1 = total_k;
+  const int64_t v0 = r0 * row_vecs, v1 = r1 * row_vecs;
+  for (int64_t i = v0 + (int64_t)blockIdx.y * 256 + threadIdx.x; i < v1; i += (int64_t)gridDim.y * 256) {
+    dk[i] = u32x4{0, 0, 0, 0};
+    dv[i] = u32x4{0, 0, 0, 0};
+  }
+}
+
 __global__ __launch_bounds__(256) void fill_zero_kernel(u32x4 *__restrict__ p, int64_t nvec) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -72,10 +88,11 @@ __global__ __launch_bounds__(256) void cvt_elem_kernel(const float *__restrict__
 struct BwdWorkspace {
   int64_t sched_kv, sched_q, delta, lse2, dk_acc, dv_acc, total;
 };
+// acc: with the fp32 dK/dV accumulators (needed only when key blocks are cut into pieces)
 BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias) {
   BwdWorkspace w;
   int64_t o = 0;
-  w.sched_kv = o; o += sched_region_bytes(p->num_tasks, bwd_max_items(p));
+  w.sched_kv = o; o += sched_shared_region_bytes(p->num_tasks, bwd_max_items(p));
   w.sched_q = o; o += sched_region_bytes(p->num_tasks, dq_max_items(p));
   w.delta = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.lse2 = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
@@ -102,8 +119,9 @@ extern "C" int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p) {
   if (!p) return fail(DISTCA_E_INVALID, "bwd_workspace_bytes: null params");
   int rc = validate_params(p);
   if (rc) return rc;
-  // sized for the aliased-KV form so one query serves both call shapes
-  return bwd_layout(p, true).total;
+  // the work lists and row statistics, and, only when key blocks are cut into pieces (small batches whose caller
+  // allows float atomics), the fp32 dK/dV accumulators
+  return bwd_layout(p, bwd_split_target(p) > 0).total;
 }
 
 extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
@@ -148,16 +166,16 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   int rc = validate_params(p);
   if (rc) return rc;
   const bool alias = kv_off != nullptr;
-  if (p->deterministic && alias)
-    return fail(DISTCA_E_UNSUPPORTED, "ca_bwd: deterministic=1 with kv_task_offsets (dK/dV of aliased rows are summed with float atomics)");
   if (!dout || !q || !k || !v || !out || (!qs.lse && !qs.lse_tok) || !dq || !dk || !dv || !cu_q || !cu_k) {
     if (p->num_tasks == 0 || (p->total_q == 0 && p->total_k == 0)) return DISTCA_OK;
     return fail(DISTCA_E_INVALID, "ca_bwd: null pointer");
   }
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
     return fail(DISTCA_E_INVALID, "ca_bwd: tensors must be 16-byte aligned");
-  // dK/dV go through fp32 accumulators when tasks alias K/V rows or when key blocks are cut into pieces
-  const bool use_acc = alias || bwd_split_target(p) > 0;
+  // dK/dV go through fp32 accumulators (float atomics) only when key blocks are cut into pieces.  Tasks over shared
+  // K/V rows otherwise have one work item per (group of tasks, key block), which sums in registers like any other.
+  const bool use_acc = bwd_split_target(p) > 0;
+  const bool shared = alias && !use_acc;
   const BwdWorkspace w = bwd_layout(p, use_acc);
   if (!workspace || workspace_bytes < w.total)
     return fail(DISTCA_E_WORKSPACE, "ca_bwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)w.total);
@@ -175,9 +193,10 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     } else if (p->num_tasks == 0 || p->total_q == 0) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dk, kv_elems / 8);
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dv, kv_elems / 8);
-    } else {
+    } else if (!shared) {
       // every task owns its rows and the dK/dV kernel writes each row of a task that has queries exactly once:
-      // only the others need the fill (at 131 072 tokens that is 0.5 GB of writes not made)
+      // only the others need the fill (at 131 072 tokens that is 0.5 GB of writes not made); with shared rows the
+      // fill follows the list builder below, which finds the rows no group of tasks covers
       hipLaunchKernelGGL(fill_unowned_rows_kernel, dim3((unsigned)p->num_tasks + 1, 16), dim3(256), 0, s, (u32x4 *)dk, (u32x4 *)dv,
                          cu_q, cu_k, p->num_tasks, p->total_k, (int64_t)p->num_heads_kv * kHeadDim / 8);
     }
@@ -194,6 +213,7 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   a.dk_acc = use_acc ? (float *)(ws + w.dk_acc) : nullptr;
   a.dv_acc = use_acc ? (float *)(ws + w.dv_acc) : nullptr;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
+  a.grp_first = a.grp_tasks = a.grp_off = a.grp_lmax = nullptr;
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
@@ -219,12 +239,22 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   }
   // ---- dK, dV: one workgroup per (task, 256-key block, kv head)
   {
-    const SchedGeom geom = bwd_geom(p);
     const int64_t max_items = bwd_max_items(p);
-    rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_kv), max_items, s);
-    if (rc) return rc;
-    // the list is sized for tasks over shared K/V rows; without them the tighter bound sizes the grid (a batch of
-    // many short documents and one long one would otherwise launch mostly workgroups that find nothing to do)
+    int32_t *list = (int32_t *)(ws + w.sched_kv);
+    if (shared) {
+      rc = launch_build_shared_schedule(cu_q, cu_k, kv_off, p->num_tasks, p->total_k, bwd_shared_geom(p), list, max_items, s);
+      if (rc) return rc;
+      const SharedGroups sg = shared_groups(list, p->num_tasks, max_items);
+      a.grp_first = sg.first; a.grp_tasks = sg.tasks; a.grp_off = sg.off; a.grp_lmax = sg.lmax;
+      hipLaunchKernelGGL(fill_gap_rows_kernel, dim3((unsigned)p->num_tasks + 1, 16), dim3(256), 0, s, (u32x4 *)dk, (u32x4 *)dv,
+                         sg.gap_lo, sg.gap_hi, p->total_k, (int64_t)p->num_heads_kv * kHeadDim / 8);
+    } else {
+      rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, bwd_geom(p), list, max_items, s);
+      if (rc) return rc;
+    }
+    // when the list is sized for pieces of tasks over shared K/V rows but the tasks own their rows, the tighter bound
+    // sizes the grid (a batch of many short documents and one long one would otherwise launch mostly workgroups
+    // that find nothing to do)
     const int64_t grid_items = alias ? max_items : bwd_key_blocks_own_rows(p) + bwd_split_target(p);
     const int64_t grid = grid_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
@@ -232,7 +262,7 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
-    rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, s);
+    rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, shared, s);
     if (rc) return rc;
   }
   if (use_acc) {

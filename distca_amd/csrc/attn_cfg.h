@@ -10,8 +10,8 @@ namespace distca {
 
 constexpr int kHeadDim = 128;
 
-// Forward and dQ kernels: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles
-// of 64 keys.  One sub-tile keeps a wave under 256 registers, so a compute unit holds eight waves.
+// Forward kernel: each wave owns FWD_MSUB sub-tiles of 32 flattened query rows; KV tiles of 64 keys.  One
+// sub-tile keeps a wave under 256 registers, so a compute unit holds eight waves.
 #ifndef DISTCA_FWD_MSUB
 #define DISTCA_FWD_MSUB 1
 #endif
@@ -24,8 +24,8 @@ constexpr int kFwdRows = kFwdWaves * 32 * kFwdMsub;
 constexpr int kDqRows = 256;  // the dQ kernel: four waves of two 32-row sub-blocks
 constexpr int kFwdKV = 64;
 
-// Backward: a workgroup owns 256 keys (eight waves of 32, in two groups that work through the same
-// query blocks half a period apart); query rows are streamed in blocks of 32 flattened rows.
+// dK/dV kernel: a workgroup owns 256 keys (four waves of 64, one per SIMD); query rows are streamed in blocks of
+// 32 flattened rows.
 constexpr int kBwdRows = 32;
 constexpr int kBwdKV = 256;
 
@@ -103,12 +103,26 @@ inline int64_t dq_max_items(const distca_ca_params *p) {
   return (int64_t)p->total_q * group / kDqRows + p->num_tasks + 1;
 }
 inline int64_t bwd_max_items(const distca_ca_params *p) {
-  // cutting adds at most total cost / piece <= split_target pieces to the key blocks (piece_size rounds up)
-  return bwd_key_blocks_bound(p) + bwd_split_target(p);
+  // Without cutting, items are (task, key block) over rows the task owns, or (group of tasks that share rows, key
+  // block): either way the blocks tile stored rows.  With cutting (small batches only) tasks over shared rows have an
+  // item per task and key block, and cutting adds at most total cost / piece <= split_target pieces (piece_size rounds up).
+  const int32_t split = bwd_split_target(p);
+  return split > 0 ? bwd_key_blocks_bound(p) + split : bwd_key_blocks_own_rows(p);
+}
+// The dK/dV list over groups of tasks that share stored K/V rows: an item's cost is the sum over the group's tasks.
+inline SchedGeom bwd_shared_geom(const distca_ca_params *p) {
+  SchedGeom g = bwd_geom(p);
+  g.split_target = 0;
+  g.cost_shift = pick_cost_shift((int64_t)p->total_q * g.group / kBwdRows + p->num_tasks + 1);
+  return g;
 }
 
 int launch_build_schedule(int kind, const int32_t *cu_q, const int32_t *cu_k, int32_t num_tasks, const SchedGeom &g,
                           int32_t *ws, int64_t max_items, hipStream_t stream);
+// The dK/dV list over groups of tasks that share stored K/V rows (sched.h, SharedGroups); the region behind `ws` is
+// sched_shared_region_bytes long.
+int launch_build_shared_schedule(const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off, int32_t num_tasks, int32_t total_k,
+                                 const SchedGeom &g, int32_t *ws, int64_t max_items, hipStream_t stream);
 
 inline int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 

@@ -157,6 +157,40 @@ DISTCA_HD int64_t sched_region_bytes(int32_t num_tasks, int64_t max_items) {
   return sched_ticket_off(num_tasks, max_items) + kTicketBytes;
 }
 
+// The dK/dV list of a batch whose tasks share stored K/V rows (kv_task_offsets) is made over groups: the tasks
+// (with queries) that start at one stored row read prefixes of one stored document, and a work item
+// (group, key block) walks the query blocks of every task of the group whose prefix holds the block, so that the
+// block's dK/dV are summed in registers and written once: no atomics, no accumulators in memory, the same bits in
+// every run.  Tasks that start at different rows must not share rows (the builder counts the groups that run into
+// the next one in word 3 of the list's header).  Behind the ticket counters the region then holds, all int32:
+//   first [B + 1]   group u's tasks are tasks[first[u] .. first[u + 1]), by (prefix length, task index)
+//   tasks [B]
+//   off   [B]       first stored row of the group        lmax [B]   its longest prefix
+//   gap_lo, gap_hi [B + 1]   stored rows [gap_lo[u], gap_hi[u]) belong to no group (zeroed by the backward): from the
+//                            end of group u to the start of the next one; entry `number of groups`: the rows before
+//                            the first group
+//   tmp   [2 B]     scratch of the builder
+struct SharedGroups {
+  int32_t *first, *tasks, *off, *lmax, *gap_lo, *gap_hi, *tmp;
+};
+DISTCA_HD int64_t shared_groups_ints(int32_t num_tasks) { return ((int64_t)8 * ((int64_t)num_tasks + 1) + 63) / 64 * 64; }
+DISTCA_HD int64_t sched_shared_region_bytes(int32_t num_tasks, int64_t max_items) {
+  return sched_region_bytes(num_tasks, max_items) + shared_groups_ints(num_tasks) * (int64_t)sizeof(int32_t);
+}
+DISTCA_HD SharedGroups shared_groups(int32_t *ws, int32_t num_tasks, int64_t max_items) {
+  int32_t *p = ws + sched_region_bytes(num_tasks, max_items) / (int64_t)sizeof(int32_t);
+  const int64_t b = num_tasks;
+  SharedGroups g;
+  g.first = p;
+  g.tasks = p + (b + 1);
+  g.off = p + (2 * b + 1);
+  g.lmax = p + (3 * b + 1);
+  g.gap_lo = p + (4 * b + 1);
+  g.gap_hi = p + (5 * b + 2);
+  g.tmp = p + (6 * b + 3);
+  return g;
+}
+
 #if defined(__HIPCC__)
 // Draws this workgroup's (item rank, kv head); false when every list is used up.  `slot` is two ints
 // of LDS that the caller may reuse afterwards.  All threads of the workgroup must call it.

@@ -402,14 +402,16 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
 
     With `in_place` (the default, for head counts that keep the q part of a request token 16-byte
     aligned) the kernels read dO, O, lse and q where they lie in the receive buffer and write dq
-    where it belongs in the send buffer; K and V are unpacked, dk and dv summed and packed as
-    before.  Returns (None, dk, dv) then, else (dq, dk, dv).  Both leave the same bytes in the send
+    where it belongs in the send buffer; K and V are unpacked (with `meta.shared_kv` every stored shard once, and
+    dk / dv then come out summed over the tasks that read a shard and are packed once), dk and dv otherwise summed
+    over the duplicate copies and packed as before.  Returns (None, dk, dv) then, else (dq, dk, dv).  Both leave the same bytes in the send
     buffer."""
     dev = recv_buffer.device
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
     in_place = in_place and (hq * 4) % 16 == 0 and dtype in _ELEM_CODE and d == HEAD_DIM
-    # summed dK/dV of shared rows come from float atomics: not when the caller insists on a deterministic backward
-    shared = meta.shared_kv if in_place and not fa_args.deterministic else None
+    # one copy of every K/V shard, whatever the deterministic switch says: one work item per (document, key block)
+    # sums dK/dV over the document's tasks in registers
+    shared = meta.shared_kv if in_place else None
     k_rows = shared.num_rows if shared is not None else meta.k_shape[0]
     recv_k = torch.empty((k_rows, meta.k_shape[1]), dtype=dtype, device=dev)
     recv_v = torch.empty_like(recv_k)

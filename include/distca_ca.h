@@ -120,6 +120,10 @@ int distca_grad_sum(void *data, int dtype, const int32_t *num_copies,
  * Task b: query rows q[cu_seqlens_q[b] .. cu_seqlens_q[b+1]) (Lq rows) attend
  * to key/value rows k[ks .. ks+Lk) with Lk = cu_seqlens_k[b+1]-cu_seqlens_k[b]
  * and ks = kv_task_offsets ? kv_task_offsets[b] : cu_seqlens_k[b].  With
+ * kv_task_offsets, tasks that start at the same row read prefixes of one stored
+ * document (the reference materialises one copy of the prefix per task,
+ * compute_metadata.py:429-448); tasks that start at different rows must not
+ * share rows, and ks + Lk <= total_k.  With
  * causal != 0 row i sees column j iff j <= i + (Lk - Lq) (bottom-right
  * aligned, the flash-attn 2.1+ convention the reference relies on at
  * per_doc_cp_attn.py:326,406-411).  q-head h reads kv-head h / (Hq/Hkv).
@@ -150,8 +154,12 @@ typedef struct distca_ca_params {
   int32_t max_seqlen_k; /* upper bound of any task's Lk                       */
   float softmax_scale;  /* multiplies q.k before softmax                      */
   int32_t causal;       /* 0 / 1                                              */
-  int32_t deterministic;/* backward only: 1 = refuse any path that uses float
-                           atomics (only the kv_task_offsets form does)       */
+  int32_t deterministic;/* backward only: 1 = use no float atomics, so that two
+                           runs give the same bits (the reference's server
+                           default, fused_comm_attn.py:95-104).  0 allows them
+                           where they pay: a batch too small to occupy the
+                           device has its key blocks cut into pieces whose
+                           dK/dV are added up with atomics                    */
   int32_t dtype;        /* element type of q, k, v, out and the gradients:
                            DISTCA_DTYPE_BF16 or DISTCA_DTYPE_F16; 0 (callers
                            written before the field existed) means bf16      */
@@ -160,7 +168,8 @@ typedef struct distca_ca_params {
 /* Size of the workspace an attention call needs (no reference counterpart: flash-attn
  * allocates its own).  The workspace holds the work list the call builds on the device
  * and the counters its workgroups draw their work from (and, in the backward, the row
- * statistics and the fp32 accumulators of aliased K/V rows); its contents are rewritten
+ * statistics: 8 bytes per query row and head; fp32 dK/dV accumulators only for a small
+ * batch with deterministic == 0, whose key blocks are cut into pieces); its contents are rewritten
  * by every call, so calls that may run at the same time on different streams each need
  * a workspace of their own, while calls ordered on one stream can share one.           */
 int64_t distca_ca_fwd_workspace_bytes(const distca_ca_params *p);
@@ -215,9 +224,13 @@ int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off,
                          int64_t workspace_bytes, void *stream);
 
 /* dk/dv rows are written once per task when kv_task_offsets is NULL.  When it
- * is given, tasks may alias KV rows and dk/dv hold the sum over every task
- * that read the row (what the reference obtains with duplicated KV copies and
- * inplace_grad_sum_kernel). */
+ * is given, dk/dv of a stored row hold the sum over every task that read the
+ * row (what the reference obtains with duplicated KV copies and
+ * inplace_grad_sum_kernel, csrc/core/memcpy.cu:158-236): one work item per
+ * (stored document, block of 256 keys) walks the query rows of every task whose
+ * prefix holds the block, sums in registers and writes the rows once, so the
+ * result is the same in every run whatever `deterministic` says; rows that no
+ * task reads come back as zeros. */
 int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v,
                   const void *out, const float *lse, void *dq, void *dk,
                   void *dv, const int32_t *cu_seqlens_q,

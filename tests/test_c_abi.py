@@ -137,17 +137,42 @@ def test_attention_argument_errors_are_reported_before_any_launch():
     assert lib.distca_ca_fwd(*args(q=odd)) == -1
     assert b"aligned" in lib.distca_last_error()
     assert lib.distca_ca_fwd(*args(q=None)) == -1
-    # backward: deterministic together with shared KV rows is refused, as documented
+    # backward: deterministic together with shared KV rows is served (one work item owns a key block on behalf of every
+    # task that reads it), so the call passes validation up to the workspace check, like the form without kv_task_offsets
     pd = _p(deterministic=1)
     needb = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(pd))
-    bargs = [ptr] * 9 + [ptr, ptr, ptr, ctypes.byref(pd), ptr, needb, None]
-    assert lib.distca_ca_bwd(*bargs) == -2
-    assert b"deterministic" in lib.distca_last_error()
-    bargs[11] = None                                          # no kv_task_offsets: passes validation up to the workspace check
-    bargs[14] = 64                                             # (the size query covers the shared-KV form; 64 B is too small for either)
+    bargs = [ptr] * 9 + [ptr, ptr, ptr, ctypes.byref(pd), ptr, 64, None]
     assert lib.distca_ca_bwd(*bargs) == -3
+    assert b"workspace" in lib.distca_last_error()
+    bargs[11] = None
+    assert lib.distca_ca_bwd(*bargs) == -3
+    bargs[14] = needb
+    bargs[0] = odd
+    assert lib.distca_ca_bwd(*bargs) == -1
+    assert b"aligned" in lib.distca_last_error()
     # a batch without tasks or rows is a no-op that touches nothing
     assert lib.distca_ca_fwd(None, None, None, None, None, None, None, None, ctypes.byref(_p(num_tasks=0, total_q=0, total_k=0)), None, 0, None) == 0
+
+
+def test_backward_workspace_is_sized_for_what_the_call_needs():
+    """The work lists and the two row statistics, and nothing else, for a batch large enough to occupy the device or a
+    deterministic one: 131072 tokens with 32 query heads need 34 MB.  Only a small batch whose caller allows float
+    atomics (its key blocks are then cut into pieces) also brings the fp32 dK/dV accumulators."""
+    lib = _lib.load()
+    big = _p(num_tasks=27, total_q=131072, total_k=131072, num_heads_q=32, num_heads_kv=8, max_seqlen_q=65536, max_seqlen_k=65536)
+    n = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(big))
+    stats = 2 * 32 * 131072 * 4
+    assert stats < n <= 40e6
+    big.deterministic = 1
+    assert lib.distca_ca_bwd_workspace_bytes(ctypes.byref(big)) == n
+    cfg5 = _p(num_tasks=40, total_q=524288, total_k=524288, num_heads_q=64, num_heads_kv=8, max_seqlen_q=262144, max_seqlen_k=262144)
+    assert lib.distca_ca_bwd_workspace_bytes(ctypes.byref(cfg5)) <= 2 * 64 * 524288 * 4 + 8e6
+    small = _p(num_tasks=3, total_q=4096, total_k=4096, num_heads_q=32, num_heads_kv=8, max_seqlen_q=2560, max_seqlen_k=2560)
+    pieces = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(small))
+    small.deterministic = 1
+    whole = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(small))
+    assert pieces - whole >= 2 * 4096 * 8 * 128 * 4          # the two accumulators
+    assert whole < 2 * 32 * 4096 * 4 + 1e6
 
 
 def test_python_wrappers_reject_wrong_inputs():

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, total_k=None, bwd=True, d=128, kv_grad_tol=None,
-         dtype=torch.bfloat16):
+         dtype=torch.bfloat16, deterministic=False):
     from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
     cu_q, cu_k = cu(q_lens), cu(k_lens)
     tq = int(cu_q[-1])
@@ -36,9 +36,14 @@ def _run(q_lens, k_lens, hq, hkv, seed, cuda, causal=True, kv_offsets=None, tota
     ref_dq, ref_dk, ref_dv = ca_reference_bwd(do, q, k, v, cu_q, cu_k, causal=causal, kv_task_offsets=kv_offsets,
                                               out=out.cpu(), softmax_lse=lse.cpu())
     dq, dk, dv = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal,
-                               False, dkv)
+                               deterministic, dkv)
     torch.cuda.synchronize()
     assert dq.dtype == dk.dtype == dv.dtype == dtype and dq.shape == qd.shape and dk.shape == kd.shape
+    if deterministic:
+        again = ca_varlen_bwd(dod, qd, kd, vd, out, lse, dcu_q, dcu_k, int(max(q_lens)), int(max(k_lens)), None, causal, True, dkv)
+        torch.cuda.synchronize()
+        for name, x, y in zip(("dq", "dk", "dv"), (dq, dk, dv), again):
+            assert torch.equal(x, y), f"{name} differs between two deterministic runs"
     assert_close_bf16(dq, ref_dq, "dq")
     tol = dict(max_abs=kv_grad_tol[0], mean_rel=kv_grad_tol[1]) if kv_grad_tol else {}
     assert_close_bf16(dk, ref_dk, "dk", **tol)
@@ -89,6 +94,36 @@ def test_prefix_lengths_around_tile_and_ring_boundaries(cuda, hq, hkv):
 def test_shared_kv_prefix(cuda):
     """Three shards of one 600-token document reading one stored KV copy."""
     _run([200, 150, 250], [200, 350, 600], 8, 2, 5, cuda, kv_offsets=[0, 0, 0], total_k=600)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4), (12, 4)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_shared_kv_documents_deterministic(cuda, hq, hkv, causal):
+    """Three stored documents read by tasks that are prefixes of them, with the deterministic switch the reference's
+    server has by default: one work item per (document, key block) walks the query rows of every task that sees the
+    block and writes dK/dV once.  The documents lie in the store out of order and with unread rows before, between
+    and behind them (those come back as zeros); prefixes end around key-block (256) and tile (32, 64) edges, one task
+    has no queries, one document is read by a single task, two tasks of a document have the same prefix length."""
+    #          document at row 40 (700 rows)      at row 1000 (513 rows)   at row 800 (130 rows)
+    k_lens = [255, 256, 257, 700, 700, 33,        512, 513, 300,            130]
+    q_lens = [255, 1, 1, 443, 100, 33,            212, 1, 0,                64]
+    offs = [40, 40, 40, 40, 40, 40,               1000, 1000, 1000,         800]
+    _run(q_lens, k_lens, hq, hkv, 31, cuda, causal=causal, kv_offsets=offs, total_k=1600, deterministic=True)
+
+
+def test_queries_that_see_no_key(cuda):
+    """A task with more queries than keys under the bottom-right aligned mask: its first Lq - Lk rows see nothing.
+    Their output and dq are zero and their lse is -inf, and they add nothing to dk / dv (the backward kernels meet
+    exp2(+inf) for such rows and must mask it away)."""
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    _run([300, 64], [100, 64], 8, 2, 41, cuda)
+    q, k, v, do = (t.to(cuda) for t in make_qkv(364, 164, 8, 2, 128, 41))
+    cq, ck = torch.tensor(cu([300, 64]), device=cuda), torch.tensor(cu([100, 64]), device=cuda)
+    out, lse = ca_varlen_fwd(q, k, v, cq, ck, 300, 100)
+    dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cq, ck, 300, 100)
+    torch.cuda.synchronize()
+    assert (out[:200] == 0).all() and (dq[:200] == 0).all() and torch.isinf(lse[:, :200]).all() and (lse[:, :200] < 0).all()
+    assert torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all() and torch.isfinite(dq.float()).all()
 
 
 def test_non_causal(cuda):
