@@ -168,7 +168,7 @@ def pack_unpack_bench(torch, dev, iters: int = 10):
     return res
 
 
-def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 3, shard_cap: int = 4096):
+def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap: int = 4096):
     """The CA server's ticks on the bench workload: every document cut into shards of at most `shard_cap`
     tokens, one CA task per shard reading its document's prefix.  Forward tick = unpack K/V (each stored shard
     once) + attention reading q from the receive buffer and writing [out | lse] tokens into the send buffer;
@@ -213,8 +213,26 @@ def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 3, shard_cap:
     fill(recv, flat(q), False)
     res = {"tasks": int(plan.q_seqlens.numel()), "documents": len(docs), "shard_cap": shard_cap,
            "stored_kv_rows": T, "kv_rows_one_copy_per_task": plan.num_kv_tokens}
-    fa_det, fa_sum = FlashAttnArgs(hq, hkv, d, deterministic=True), FlashAttnArgs(hq, hkv, d, deterministic=False)
-    res["forward_ms"] = round(timed(lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det)), 3)
+    from distca_amd import _lib
+    fa_det = FlashAttnArgs(hq, hkv, d, deterministic=True)      # the reference's server default (fused_comm_attn.py:95-104)
+
+    def timed_with_kernels(fn, timers):
+        """(tick time, time of the attention kernels inside it), both per tick, over the same `iters` ticks."""
+        fn()
+        torch.cuda.synchronize()
+        _lib.timing_enable(True)
+        for t in timers:
+            _lib.timing_read(t)
+        total = timed(fn)
+        kern = sum(_lib.timing_read(t)[0] for t in timers) / (iters + 1)     # timed() warms up once more
+        _lib.timing_enable(False)
+        return round(total, 3), round(kern, 3)
+
+    fwd_timers, bwd_timers = (_lib.TIMER_CA_FWD,), (_lib.TIMER_CA_BWD_DQ, _lib.TIMER_CA_BWD)
+    res["forward_ms"], res["forward_attention_kernel_ms"] = timed_with_kernels(
+        lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det), fwd_timers)
+    res["forward_kv_unpacked_ms"], res["forward_kv_unpacked_attention_kernel_ms"] = timed_with_kernels(
+        lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det, kv_shards_in_place=False), fwd_timers)
     out, lse = ca_server_forward(recv, send, fmeta, fa_params, fa_det, in_place=False)
     del recv, send
     request = TokenLayout.of([flat(do), out, lse.T.contiguous(), flat(q)]).merge([flat(do), out, lse.T.contiguous(), flat(q)])
@@ -223,12 +241,16 @@ def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 3, shard_cap:
     fill(recv, request, True)
     del request
     send = torch.zeros(b_send, dtype=torch.uint8, device=dev)
-    bwd = lambda fa: ca_server_backward(recv, send, bmeta, fa, fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
-                                        fa_params.max_seqlen_q, fa_params.max_seqlen_kv)
-    res["backward_ms"] = round(timed(lambda: bwd(fa_sum)), 3)
-    res["backward_deterministic_ms"] = round(timed(lambda: bwd(fa_det)), 3)
-    res["note"] = ("backward_ms: one stored copy per K/V shard, dk / dv summed over tasks by float atomics; "
-                   "backward_deterministic_ms: one K/V prefix copy per task, duplicate gradients summed in copy order")
+    bwd = lambda **kw: ca_server_backward(recv, send, bmeta, fa_det, fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
+                                          fa_params.max_seqlen_q, fa_params.max_seqlen_kv, **kw)
+    res["backward_ms"], res["backward_attention_kernels_ms"] = timed_with_kernels(lambda: bwd(), bwd_timers)
+    res["backward_kv_unpacked_ms"], res["backward_kv_unpacked_attention_kernels_ms"] = timed_with_kernels(
+        lambda: bwd(kv_shards_in_place=False), bwd_timers)
+    res["note"] = ("deterministic ticks (the reference's default).  forward_ms / backward_ms: everything in place: query and "
+                   "request tokens and K/V shards read where they lie in the receive buffer, [out | lse], dq and the shards' "
+                   "dk / dv written where they belong in the send buffer, no pack kernel; *_kv_unpacked_ms: every stored K/V "
+                   "shard unpacked once into a tensor first, dk / dv packed afterwards; *_attention_kernel(s)_ms: the attention "
+                   "kernels' own share of the tick above it, by events around them")
     return res
 
 
@@ -339,8 +361,10 @@ def main():
     tick = None
     if not args.no_tick:
         tick = server_tick_bench(torch, dev, batch, q, k, v, do)
-        log(f"  server tick over {tick['tasks']} tasks: forward {tick['forward_ms']} ms, backward {tick['backward_ms']} ms "
-            f"(deterministic {tick['backward_deterministic_ms']} ms)")
+        log(f"  server tick over {tick['tasks']} tasks: forward {tick['forward_ms']} ms (kernel {tick['forward_attention_kernel_ms']}; "
+            f"K/V unpacked first: {tick['forward_kv_unpacked_ms']}, kernel {tick['forward_kv_unpacked_attention_kernel_ms']}), "
+            f"backward {tick['backward_ms']} ms (kernels {tick['backward_attention_kernels_ms']}; K/V unpacked first: "
+            f"{tick['backward_kv_unpacked_ms']}, kernels {tick['backward_kv_unpacked_attention_kernels_ms']})")
 
     cpu = None
     if args.cpu_seconds > 0:

@@ -13,7 +13,7 @@ from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int6
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdistca_ca.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class CaParams(Structure):
@@ -32,6 +32,14 @@ class PackJob(Structure):
     _fields_ = [
         ("tensor", c_void_p), ("seq_offset", c_void_p), ("seq_tokens", c_void_p), ("copy_seq_mask", c_void_p),
         ("num_seq", c_int64), ("token_bytes", c_int64), ("num_tokens", c_int64),
+    ]
+
+
+class KvShards(Structure):
+    """struct distca_kv_shards (include/distca_ca.h)."""
+    _fields_ = [
+        ("num_shards", c_int32), ("row_start", c_void_p), ("k_offset", c_void_p), ("v_offset", c_void_p),
+        ("task_shard", c_void_p), ("dk_offset", c_void_p), ("dv_offset", c_void_p),
     ]
 
 
@@ -54,6 +62,10 @@ SYMBOLS = {
                                       POINTER(CaParams), c_void_p]),
     "distca_ca_fwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                      c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_fwd_buffers": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, POINTER(KvShards), c_void_p, c_void_p, c_int64,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
+    "distca_ca_bwd_buffers": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, POINTER(KvShards), c_void_p, c_void_p, c_int64,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd": (c_int, [c_void_p] * 9 + [c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),
     "distca_ca_bwd_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, POINTER(CaParams), c_void_p, c_int64, c_void_p]),

@@ -103,4 +103,4 @@ extern "C" int distca_timing_read(int which, double *total_ms, int64_t *launches
 }
 
 extern "C" const char *distca_last_error(void) { return distca::error_buffer(); }
-extern "C" int distca_abi_version(void) { return 3; }
+extern "C" int distca_abi_version(void) { return 4; }

@@ -5,6 +5,7 @@
 
 #include "../../include/distca_ca.h"
 #include "common.h"
+#include "kv_shards.h"
 
 namespace distca {
 
@@ -22,6 +23,7 @@ struct BwdArgs {
   const int32_t *cu_q, *cu_k, *kv_off;
   // the dK/dV list over groups of tasks that share stored K/V rows (sched.h, SharedGroups); null otherwise
   const int32_t *grp_first, *grp_tasks, *grp_off, *grp_lmax;
+  KvShards shards;  // kernels that read K/V in place: k, v, dk, dv are then the bases the shards' offsets count from
   const int32_t *sched;
   int32_t *tickets;  // one counter per kv head (sched.h)
   const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
@@ -50,17 +52,24 @@ struct BwdQuerySide {
   int64_t dq_tok_bytes;
 };
 // The backward behind distca_ca_bwd and distca_ca_bwd_tokens, per element type (attn_bwd.hip compiled for each).
+// kv_shards: null, or the table through which K/V rows are read and dK/dV rows written in place (kv_shards.h)
 int run_bwd(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
-            const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+            const int32_t *kv_off, const distca_kv_shards *kv_shards, const distca_ca_params *p, void *workspace,
+            int64_t workspace_bytes, void *stream);
 int run_bwd_f16(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
-                const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+                const int32_t *kv_off, const distca_kv_shards *kv_shards, const distca_ca_params *p, void *workspace,
+                int64_t workspace_bytes, void *stream);
 // The forward behind distca_ca_fwd_tokens, per element type (attn_fwd.hip compiled for each).
-int run_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v, void *out_base,
-                   const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q, const int32_t *cu_k,
-                   const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
-int run_fwd_tokens_f16(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v, void *out_base,
-                       const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q, const int32_t *cu_k,
-                       const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream);
+int run_fwd_tokens(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v,
+                   const distca_kv_shards *kv_shards, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes, float *lse,
+                   const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
+                   int64_t workspace_bytes, void *stream);
+int run_fwd_tokens_f16(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v,
+                       const distca_kv_shards *kv_shards, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes, float *lse,
+                       const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
+                       int64_t workspace_bytes, void *stream);
+// Checks a table of shards (host-visible fields only) and turns it into the kernels' form.
+int make_kv_shards(const distca_kv_shards *in, const int32_t *kv_off, bool backward, KvShards *out);
 
 // The dK/dV kernel with 64 keys per wave (attn_bwd_dkdv64.hip): LDS bytes it needs, and its launch.
 int dkdv64_lds_bytes();

@@ -68,6 +68,24 @@ __global__ __launch_bounds__(256) void fill_gap_rows_kernel(u32x4 *__restrict__ 
   }
 }
 
+// The same with the dK/dV rows addressed through a table of shards (kv_shards.h): one row per 128-thread slice.
+__global__ __launch_bounds__(256) void fill_gap_rows_shards_kernel(uint8_t *__restrict__ dk, uint8_t *__restrict__ dv,
+                                                                  const int32_t *__restrict__ gap_lo, const int32_t *__restrict__ gap_hi,
+                                                                  int32_t total_k, int64_t row_bytes, KvShards sh) {
+  int64_t r0 = gap_lo[blockIdx.x], r1 = gap_hi[blockIdx.x];
+  if (r0 < 0) r0 = 0;
+  if (r1 > total_k) r1 = total_k;
+  for (int64_t r = r0 + blockIdx.y; r < r1; r += gridDim.y) {
+    const int s = find_shard(sh.row_start, sh.num_shards, (int)r);
+    const int64_t in_shard = (r - sh.row_start[s]) * row_bytes;
+    u32x4 *pk = reinterpret_cast<u32x4 *>(dk + sh.dk_off[s] + in_shard), *pv = reinterpret_cast<u32x4 *>(dv + sh.dv_off[s] + in_shard);
+    for (int64_t i = threadIdx.x; i < row_bytes / 16; i += 256) {
+      pk[i] = u32x4{0, 0, 0, 0};
+      pv[i] = u32x4{0, 0, 0, 0};
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void fill_zero_kernel(u32x4 *__restrict__ p, int64_t nvec) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -88,11 +106,11 @@ __global__ __launch_bounds__(256) void cvt_elem_kernel(const float *__restrict__
 struct BwdWorkspace {
   int64_t sched_kv, sched_q, delta, lse2, dk_acc, dv_acc, total;
 };
-// acc: with the fp32 dK/dV accumulators (needed only when key blocks are cut into pieces)
-BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias) {
+// acc: with the fp32 dK/dV accumulators (needed only when key blocks are cut into pieces); max_items_kv: room of the dK/dV list
+BwdWorkspace bwd_layout(const distca_ca_params *p, bool alias, int64_t max_items_kv) {
   BwdWorkspace w;
   int64_t o = 0;
-  w.sched_kv = o; o += sched_shared_region_bytes(p->num_tasks, bwd_max_items(p));
+  w.sched_kv = o; o += sched_shared_region_bytes(p->num_tasks, max_items_kv);
   w.sched_q = o; o += sched_region_bytes(p->num_tasks, dq_max_items(p));
   w.delta = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
   w.lse2 = o; o += align_up((int64_t)p->num_heads_q * p->total_q * 4, 256);
@@ -121,7 +139,7 @@ extern "C" int64_t distca_ca_bwd_workspace_bytes(const distca_ca_params *p) {
   if (rc) return rc;
   // the work lists and row statistics, and, only when key blocks are cut into pieces (small batches whose caller
   // allows float atomics), the fp32 dK/dV accumulators
-  return bwd_layout(p, bwd_split_target(p) > 0).total;
+  return bwd_layout(p, bwd_split_target(p) > 0, bwd_max_items(p)).total;
 }
 
 extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out, const float *lse,
@@ -130,13 +148,24 @@ extern "C" int distca_ca_bwd(const void *dout, const void *q, const void *k, con
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
   const int64_t row_bytes = (int64_t)p->num_heads_q * kHeadDim * 2;
   const BwdQuerySide qs{dout, q, out, lse, nullptr, nullptr, row_bytes, dq, nullptr, row_bytes};
-  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, nullptr, p, workspace, workspace_bytes, stream);
 }
 
 extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off, int64_t req_tok_bytes, const void *k,
                                     const void *v, void *dq_base, const int64_t *dq_task_off, int64_t dq_tok_bytes, void *dk,
                                     void *dv, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
                                     const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+  return distca_ca_bwd_buffers(req_base, req_task_off, req_tok_bytes, k, v, nullptr, dq_base, dq_task_off, dq_tok_bytes, dk, dv, cu_q,
+                               cu_k, kv_off, p, workspace, workspace_bytes, stream);
+}
+
+// kv_shards may be null here (distca_ca_bwd_tokens comes through this function); the public contract of the name
+// requires it, which the header says.
+extern "C" int distca_ca_bwd_buffers(const void *req_base, const int64_t *req_task_off, int64_t req_tok_bytes, const void *k,
+                                     const void *v, const distca_kv_shards *kv_shards, void *dq_base, const int64_t *dq_task_off,
+                                     int64_t dq_tok_bytes, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
+                                     const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes,
+                                     void *stream) {
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
   int rc = validate_params(p);
   if (rc) return rc;
@@ -153,13 +182,14 @@ extern "C" int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_tas
   // [dO | O | lse | q | pad]
   const BwdQuerySide qs{r, r ? r + 2 * row_bytes + lse_bytes : nullptr, r ? r + row_bytes : nullptr, nullptr,
                         r ? r + 2 * row_bytes : nullptr, req_task_off, req_tok_bytes, dq_base, dq_task_off, dq_tok_bytes};
-  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, p, workspace, workspace_bytes, stream);
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_bwd_f16 : run_bwd)(qs, k, v, dk, dv, cu_q, cu_k, kv_off, kv_shards, p, workspace, workspace_bytes, stream);
 }
 #endif  // !DISTCA_F16
 
 namespace distca {
 int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k,
-                       const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
+                       const int32_t *kv_off, const distca_kv_shards *kv_shards, const distca_ca_params *p, void *workspace,
+                       int64_t workspace_bytes, void *stream) {
   const void *dout = qs.dout, *q = qs.q, *out = qs.out;
   void *dq = qs.dq;
   if (!p) return fail(DISTCA_E_INVALID, "ca_bwd: null params");
@@ -174,9 +204,17 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     return fail(DISTCA_E_INVALID, "ca_bwd: tensors must be 16-byte aligned");
   // dK/dV go through fp32 accumulators (float atomics) only when key blocks are cut into pieces.  Tasks over shared
   // K/V rows otherwise have one work item per (group of tasks, key block), which sums in registers like any other.
-  const bool use_acc = bwd_split_target(p) > 0;
+  // With K/V shards read in place nothing is cut (the accumulators are dense tensors over stored rows).
+  KvShards shards{};
+  if (kv_shards) {
+    rc = make_kv_shards(kv_shards, kv_off, true, &shards);
+    if (rc) return rc;
+  }
+  const int32_t split = kv_shards ? 0 : bwd_split_target(p);
+  const bool use_acc = split > 0;
   const bool shared = alias && !use_acc;
-  const BwdWorkspace w = bwd_layout(p, use_acc);
+  const int64_t max_items_kv = split > 0 ? bwd_key_blocks_bound(p) + split : bwd_key_blocks_own_rows(p);
+  const BwdWorkspace w = bwd_layout(p, use_acc, max_items_kv);
   if (!workspace || workspace_bytes < w.total)
     return fail(DISTCA_E_WORKSPACE, "ca_bwd: workspace %lld B < required %lld B", (long long)workspace_bytes, (long long)w.total);
   if (!aligned16(workspace)) return fail(DISTCA_E_INVALID, "ca_bwd: workspace must be 16-byte aligned");
@@ -190,6 +228,8 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     if (use_acc) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 2)), dim3(256), 0, s, (u32x4 *)(ws + w.dk_acc),
                          (w.total - w.dk_acc) / 16);
+    } else if ((p->num_tasks == 0 || p->total_q == 0) && kv_shards) {
+      return fail(DISTCA_E_UNSUPPORTED, "ca_bwd_buffers: a batch without tasks or queries (there is nothing to tell which rows to clear)");
     } else if (p->num_tasks == 0 || p->total_q == 0) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dk, kv_elems / 8);
       hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(kv_elems / 8)), dim3(256), 0, s, (u32x4 *)dv, kv_elems / 8);
@@ -214,6 +254,7 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   a.dv_acc = use_acc ? (float *)(ws + w.dv_acc) : nullptr;
   a.cu_q = cu_q; a.cu_k = cu_k; a.kv_off = kv_off;
   a.grp_first = a.grp_tasks = a.grp_off = a.grp_lmax = nullptr;
+  a.shards = shards;
   a.sched_items_off = (int32_t)sched_header_ints(p->num_tasks);
   a.hq = p->num_heads_q; a.hkv = p->num_heads_kv; a.group = p->num_heads_q / p->num_heads_kv;
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
@@ -239,15 +280,19 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   }
   // ---- dK, dV: one workgroup per (task, 256-key block, kv head)
   {
-    const int64_t max_items = bwd_max_items(p);
+    const int64_t max_items = max_items_kv;
     int32_t *list = (int32_t *)(ws + w.sched_kv);
     if (shared) {
       rc = launch_build_shared_schedule(cu_q, cu_k, kv_off, p->num_tasks, p->total_k, bwd_shared_geom(p), list, max_items, s);
       if (rc) return rc;
       const SharedGroups sg = shared_groups(list, p->num_tasks, max_items);
       a.grp_first = sg.first; a.grp_tasks = sg.tasks; a.grp_off = sg.off; a.grp_lmax = sg.lmax;
-      hipLaunchKernelGGL(fill_gap_rows_kernel, dim3((unsigned)p->num_tasks + 1, 16), dim3(256), 0, s, (u32x4 *)dk, (u32x4 *)dv,
-                         sg.gap_lo, sg.gap_hi, p->total_k, (int64_t)p->num_heads_kv * kHeadDim / 8);
+      if (kv_shards)
+        hipLaunchKernelGGL(fill_gap_rows_shards_kernel, dim3((unsigned)p->num_tasks + 1, 64), dim3(256), 0, s, (uint8_t *)dk,
+                           (uint8_t *)dv, sg.gap_lo, sg.gap_hi, p->total_k, (int64_t)p->num_heads_kv * kHeadDim * 2, shards);
+      else
+        hipLaunchKernelGGL(fill_gap_rows_kernel, dim3((unsigned)p->num_tasks + 1, 16), dim3(256), 0, s, (u32x4 *)dk, (u32x4 *)dv,
+                           sg.gap_lo, sg.gap_hi, p->total_k, (int64_t)p->num_heads_kv * kHeadDim / 8);
     } else {
       rc = launch_build_schedule(1, cu_q, cu_k, p->num_tasks, bwd_geom(p), list, max_items, s);
       if (rc) return rc;
@@ -255,11 +300,11 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
     // when the list is sized for pieces of tasks over shared K/V rows but the tasks own their rows, the tighter bound
     // sizes the grid (a batch of many short documents and one long one would otherwise launch mostly workgroups
     // that find nothing to do)
-    const int64_t grid_items = alias ? max_items : bwd_key_blocks_own_rows(p) + bwd_split_target(p);
+    const int64_t grid_items = alias ? max_items : bwd_key_blocks_own_rows(p) + split;
     const int64_t grid = grid_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
     if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_bwd: grid too large");
     a.sched = (const int32_t *)(ws + w.sched_kv);
-    a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, bwd_max_items(p));
+    a.zero_row = ws + w.sched_kv + sched_zero_row_off(p->num_tasks, max_items);
     a.tickets = (int32_t *)(ws + w.sched_kv + sched_ticket_off(p->num_tasks, max_items));
     ScopedTimer timer(DISTCA_TIMER_CA_BWD, s);
     rc = DISTCA_FN(launch_dkdv64)(a, grid, use_acc, shared, s);

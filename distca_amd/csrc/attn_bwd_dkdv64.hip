@@ -83,11 +83,16 @@ __device__ __forceinline__ void mfma32_vc(f32x16 &acc, elemx8 a, elemx8 b, const
 }
 
 #define DKDV_SHARED 0
+#define DKDV_SEG 0
 #include "attn_bwd_dkdv64_kernel.inc"
 #undef DKDV_SHARED
 #define DKDV_SHARED 1
 #include "attn_bwd_dkdv64_kernel.inc"
+#undef DKDV_SEG
+#define DKDV_SEG 1
+#include "attn_bwd_dkdv64_kernel.inc"
 #undef DKDV_SHARED
+#undef DKDV_SEG
 
 }  // namespace
 
@@ -100,11 +105,15 @@ int DISTCA_FN(launch_dkdv64)(const BwdArgs &a, int64_t grid, bool atomic_sums, b
     hipError_t e1 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     hipError_t e2 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     hipError_t e3 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_shared_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e3 == hipSuccess) e3 = hipFuncSetAttribute((const void *)ca_bwd_dkdv64_shards_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS", kLds);
     device_setup_done(kSlotBwdLds64);
   }
   if (shared && atomic_sums) return fail(DISTCA_E_INVALID, "ca_bwd: items over groups of tasks are never cut into pieces");
-  if (shared)
+  if (a.shards.num_shards > 0 && !shared) return fail(DISTCA_E_INVALID, "ca_bwd: K/V shards in place need tasks over shared stored rows");
+  if (shared && a.shards.num_shards > 0)
+    hipLaunchKernelGGL(ca_bwd_dkdv64_shards_kernel, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
+  else if (shared)
     hipLaunchKernelGGL(ca_bwd_dkdv64_shared_kernel, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
   else if (atomic_sums)
     hipLaunchKernelGGL((ca_bwd_dkdv64_kernel<true>), dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);

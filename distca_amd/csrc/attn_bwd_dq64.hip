@@ -69,6 +69,8 @@ __device__ __forceinline__ void mfma32_va0(f32x16 &acc, elemx8 a, accop_t b) {
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
 }
 
+// SEG: K/V rows are addressed through a table of shards (kv_shards.h) instead of as one dense tensor.
+template <bool SEG>
 __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
@@ -165,34 +167,77 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   // base that advances by one tile, per-lane offsets that never change); rows past the prefix read the zero row.
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
-  const elem_t *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
-  const elem_t *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *kbase = a.k + (SEG ? 0 : (int64_t)ks * kv_stride) + kvh * kHeadDim;
+  const elem_t *vbase = a.v + (SEG ? 0 : (int64_t)ks * kv_stride) + kvh * kHeadDim;
+  ShardCursor cur;  // SEG: the shard that holds the rows of the tile requested next
+  if constexpr (SEG) cur.open(a.shards, a.shards.task_shard[task]);
   uint32_t voff[2];
 #pragma unroll
   for (int ii = 0; ii < 2; ++ii) {
     const int r = 8 * wave + 4 * ii + (lane >> 4);
     voff[ii] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
   }
+  // SEG: tiles that end at or before key run_lim lie in the present shard, key x of the prefix at kvirt / vvirt +
+  // x * kv_stride; a tile past it looks for its shard first, so that a run of tiles inside one shard is requested
+  // exactly as tiles of a dense tensor are.
+  const elem_t *kvirt = kbase, *vvirt = vbase;
+  int run_lim = SEG ? 0 : lk;
+  auto issue_whole = [&](uint32_t dst, int j) {
+    const elem_t *kt = kvirt + (int64_t)j * kKeys * kv_stride, *vt = vvirt + (int64_t)j * kKeys * kv_stride;
+    lds_direct_load16(kt, voff[0], dst);
+    lds_direct_load16(kt, voff[1], dst + 4 * kRow);
+    lds_direct_load16(vt, voff[0], dst + kTile);
+    lds_direct_load16(vt, voff[1], dst + kTile + 4 * kRow);
+  };
   auto issue_tile = [&](int stage, int j) {
     const uint32_t dst = lds0 + stage * kStageBytes + 8 * wave * kRow;
-    if ((j + 1) * kKeys <= lk) {
-      const elem_t *kt = kbase + (int64_t)j * kKeys * kv_stride, *vt = vbase + (int64_t)j * kKeys * kv_stride;
-      lds_direct_load16(kt, voff[0], dst);
-      lds_direct_load16(kt, voff[1], dst + 4 * kRow);
-      lds_direct_load16(vt, voff[0], dst + kTile);
-      lds_direct_load16(vt, voff[1], dst + kTile + 4 * kRow);
-      return;
-    }
+    if constexpr (SEG) {
+      if ((j + 1) * kKeys <= run_lim) {
+        issue_whole(dst, j);
+        return;
+      }
+      const int r0 = ks + j * kKeys;
+      cur.seek(a.shards, r0);
+      if ((j + 1) * kKeys <= lk && cur.holds(r0, kKeys)) {
+        const int64_t back = (int64_t)(cur.lo - ks) * kv_stride * 2;
+        kvirt = reinterpret_cast<const elem_t *>(static_cast<uintptr_t>(uniform_i64((int64_t)reinterpret_cast<uintptr_t>(kbase) + cur.k - back)));
+        vvirt = reinterpret_cast<const elem_t *>(static_cast<uintptr_t>(uniform_i64((int64_t)reinterpret_cast<uintptr_t>(vbase) + cur.v - back)));
+        run_lim = uniform_i32(cur.hi - ks < lk ? cur.hi - ks : lk);
+        issue_whole(dst, j);
+        return;
+      }
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii) {
-      const int r = 8 * wave + 4 * ii + (lane >> 4);
-      const int key = j * kKeys + r;
-      const int chunk = (lane & 15) ^ tile_swz(r);
-      const bool ok = key < lk;
-      const elem_t *kp = ok ? kbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
-      const elem_t *vp = ok ? vbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
-      lds_direct_load16_ptr(kp + chunk * 8, dst + 4 * ii * kRow);
-      lds_direct_load16_ptr(vp + chunk * 8, dst + kTile + 4 * ii * kRow);
+      for (int ii = 0; ii < 2; ++ii) {
+        const int r = 8 * wave + 4 * ii + (lane >> 4);
+        const int key = j * kKeys + r;
+        const int chunk = (lane & 15) ^ tile_swz(r);
+        const bool ok = key < lk;
+        const uint8_t *zero = reinterpret_cast<const uint8_t *>(a.zero_row);
+        const uint8_t *kp = ok ? reinterpret_cast<const uint8_t *>(kbase) + shard_row_offset(a.shards, cur, ks + key, 0, kv_stride * 2) : zero;
+        const uint8_t *vp = ok ? reinterpret_cast<const uint8_t *>(vbase) + shard_row_offset(a.shards, cur, ks + key, 1, kv_stride * 2) : zero;
+        lds_direct_load16_ptr(kp + chunk * 16, dst + 4 * ii * kRow);
+        lds_direct_load16_ptr(vp + chunk * 16, dst + kTile + 4 * ii * kRow);
+      }
+    } else {
+      if ((j + 1) * kKeys <= lk) {
+        const elem_t *kt = kbase + (int64_t)j * kKeys * kv_stride, *vt = vbase + (int64_t)j * kKeys * kv_stride;
+        lds_direct_load16(kt, voff[0], dst);
+        lds_direct_load16(kt, voff[1], dst + 4 * kRow);
+        lds_direct_load16(vt, voff[0], dst + kTile);
+        lds_direct_load16(vt, voff[1], dst + kTile + 4 * kRow);
+        return;
+      }
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        const int r = 8 * wave + 4 * ii + (lane >> 4);
+        const int key = j * kKeys + r;
+        const int chunk = (lane & 15) ^ tile_swz(r);
+        const bool ok = key < lk;
+        const elem_t *kp = ok ? kbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
+        const elem_t *vp = ok ? vbase + (int64_t)key * kv_stride : reinterpret_cast<const elem_t *>(a.zero_row);
+        lds_direct_load16_ptr(kp + chunk * 8, dst + 4 * ii * kRow);
+        lds_direct_load16_ptr(vp + chunk * 8, dst + kTile + 4 * ii * kRow);
+      }
     }
   };
 
@@ -401,11 +446,15 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
 
 int DISTCA_FN(launch_dq64)(const BwdArgs &a, int64_t grid, hipStream_t stream) {
   if (device_setup_pending(kSlotBwdDq64)) {
-    hipError_t e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    hipError_t e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS: %s", kLds, hipGetErrorString(e));
     device_setup_done(kSlotBwdDq64);
   }
-  hipLaunchKernelGGL(ca_bwd_dq64_kernel, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
+  if (a.shards.num_shards > 0)
+    hipLaunchKernelGGL(ca_bwd_dq64_kernel<true>, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
+  else
+    hipLaunchKernelGGL(ca_bwd_dq64_kernel<false>, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
   return DISTCA_OK;
 }
 

@@ -29,6 +29,7 @@
 #include "attn_bwd.h"
 #include "attn_cfg.h"
 #include "common.h"
+#include "kv_shards.h"
 
 namespace distca {
 namespace {
@@ -58,9 +59,11 @@ struct FwdArgs {
   const int64_t *q_task_off, *out_task_off;
   int64_t q_tok_bytes, out_tok_bytes;
   int32_t lse_in_token;  // 1: lse of (token, head) as fp32 at token + hq * 256 + h * 4 (the [out | lse] reply), 0: lse[h][token]
+  KvShards shards;       // SEG kernels: k and v are the bases of a buffer that holds the stored rows shard by shard
 };
 
-template <int MSUB>
+// SEG: K/V rows are addressed through a table of shards (kv_shards.h) instead of as one dense tensor.
+template <int MSUB, bool SEG>
 __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
@@ -136,42 +139,74 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int64_t kv_stride = (int64_t)a.hkv * kHeadDim;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
   const int uwave = __builtin_amdgcn_readfirstlane(wave);
-  const elem_t *kbase = a.k + (int64_t)ks * kv_stride + kvh * kHeadDim;
-  const elem_t *vbase = a.v + (int64_t)ks * kv_stride + kvh * kHeadDim;
+  const elem_t *kbase = a.k + (SEG ? 0 : (int64_t)ks * kv_stride) + kvh * kHeadDim;
+  const elem_t *vbase = a.v + (SEG ? 0 : (int64_t)ks * kv_stride) + kvh * kHeadDim;
+  // SEG: the shards that hold the rows of the K tile and of the V tile requested next (the K requests run a tile ahead)
+  ShardCursor kcur, vcur;
+  if constexpr (SEG) {
+    kcur.open(a.shards, a.shards.task_shard[task]);
+    vcur = kcur;
+  }
   // a wave brings kRowsW rows of a K tile or of a V tile, four rows per instruction
   constexpr int kRowsW = kFwdKV / kFwdWaves, kLdW = kRowsW / 4;
-  auto issue_rows = [&](const elem_t *base, int j, uint32_t tile_off) {
+  auto issue_rows = [&](const elem_t *base, int j, uint32_t tile_off, const ShardCursor &cur, int which) {
 #pragma unroll
     for (int i = 0; i < kLdW; ++i) {
       const int r = kRowsW * uwave + 4 * i + (lane >> 4);
       const int key = j * kFwdKV + r;
       const int chunk = (lane & 15) ^ tile_swz(r);
-      const elem_t *src = base + (int64_t)key * kv_stride;
+      const elem_t *src;
+      if constexpr (SEG) {
+        src = reinterpret_cast<const elem_t *>(reinterpret_cast<const uint8_t *>(base) +
+                                               (key < lk ? shard_row_offset(a.shards, cur, ks + key, which, kv_stride * 2) : 0));
+      } else {
+        src = base + (int64_t)key * kv_stride;
+      }
       if (key >= lk) src = reinterpret_cast<const elem_t *>(a.zero_row);
       lds_direct_load16_ptr(src + chunk * 8, lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
     }
   };
-  // Tiles that lie wholly inside the prefix (all but the last one) take a form without per-lane address
-  // arithmetic: a scalar base that advances by one tile, plus a per-lane offset that never changes.
+  // Tiles that lie wholly inside the prefix (all but the last one; SEG: and inside one shard) take a form without
+  // per-lane address arithmetic: a scalar base that advances by one tile, plus a per-lane offset that never changes.
   uint32_t voff[kLdW];
 #pragma unroll
   for (int i = 0; i < kLdW; ++i) {
     const int r = kRowsW * uwave + 4 * i + (lane >> 4);
     voff[i] = (uint32_t)((r * kv_stride + (((lane & 15) ^ tile_swz(r)) * 8)) * 2);
   }
-  auto issue_rows_fast = [&](const elem_t *base, int j, uint32_t tile_off) {
-    const elem_t *tb = base + (int64_t)j * kFwdKV * kv_stride;
+  auto issue_rows_fast = [&](const elem_t *tb, uint32_t tile_off) {
 #pragma unroll
     for (int i = 0; i < kLdW; ++i) lds_direct_load16(tb, voff[i], lds0 + tile_off + (kRowsW * uwave + 4 * i) * kRowB);
   };
-  auto issue_k = [&](int j) __attribute__((always_inline)) {
-    if ((j + 1) * kFwdKV <= lk) issue_rows_fast(kbase, j, kKOff + (j & 1) * kKTile);
-    else issue_rows(kbase, j, kKOff + (j & 1) * kKTile);
+  // Key j * kFwdKV + r of a tile that ends at or before key `lim` lies at virt + (j * kFwdKV + r) * kv_stride.  Without
+  // SEG that is the whole prefix but for its last, partial tile; with SEG the tiles inside the present shard: a tile
+  // past `lim` looks for its shard (which moves virt and lim on) and only takes the per-lane form when it straddles
+  // two shards or the end of the prefix, so that a run of tiles inside one shard costs what it costs without SEG.
+  struct Run {
+    const elem_t *virt;
+    int lim;
   };
-  auto issue_v = [&](int j) __attribute__((always_inline)) {
-    if ((j + 1) * kFwdKV <= lk) issue_rows_fast(vbase, j, kVOff + (j & 1) * kVTile);
-    else issue_rows(vbase, j, kVOff + (j & 1) * kVTile);
+  Run krun{kbase, SEG ? 0 : lk}, vrun{vbase, SEG ? 0 : lk};
+  auto issue_kv = [&](const elem_t *base, int j, uint32_t tile_off, Run &run, ShardCursor &cur, int which) __attribute__((always_inline)) {
+    if ((j + 1) * kFwdKV <= run.lim) {
+      issue_rows_fast(run.virt + (int64_t)j * kFwdKV * kv_stride, tile_off);
+      return;
+    }
+    if constexpr (SEG) {
+      const int r0 = ks + j * kFwdKV;
+      cur.seek(a.shards, r0);
+      if ((j + 1) * kFwdKV <= lk && cur.holds(r0, kFwdKV)) {
+        run.virt = reinterpret_cast<const elem_t *>(static_cast<uintptr_t>(uniform_i64(
+            (int64_t)reinterpret_cast<uintptr_t>(base) + (which ? cur.v : cur.k) - (int64_t)(cur.lo - ks) * kv_stride * 2)));
+        run.lim = uniform_i32(cur.hi - ks < lk ? cur.hi - ks : lk);
+        issue_rows_fast(run.virt + (int64_t)j * kFwdKV * kv_stride, tile_off);
+        return;
+      }
+    }
+    issue_rows(base, j, tile_off, cur, which);
   };
+  auto issue_k = [&](int j) __attribute__((always_inline)) { issue_kv(kbase, j, kKOff + (j & 1) * kKTile, krun, kcur, 0); };
+  auto issue_v = [&](int j) __attribute__((always_inline)) { issue_kv(vbase, j, kVOff + (j & 1) * kVTile, vrun, vcur, 1); };
 
   // ---- accumulators
   f32x16 oacc[MSUB][4];
@@ -463,10 +498,35 @@ extern "C" int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_of
                                     float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off,
                                     const distca_ca_params *p, void *workspace, int64_t workspace_bytes, void *stream) {
   if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
-  return (p->dtype == DISTCA_DTYPE_F16 ? run_fwd_tokens_f16 : run_fwd_tokens)(q_base, q_task_off, q_tok_bytes, k, v, out_base, out_task_off,
-                                                                              out_tok_bytes, lse, cu_q, cu_k, kv_off, p, workspace,
-                                                                              workspace_bytes, stream);
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_fwd_tokens_f16 : run_fwd_tokens)(q_base, q_task_off, q_tok_bytes, k, v, nullptr, out_base,
+                                                                              out_task_off, out_tok_bytes, lse, cu_q, cu_k, kv_off, p,
+                                                                              workspace, workspace_bytes, stream);
 }
+
+extern "C" int distca_ca_fwd_buffers(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k,
+                                     const void *v, const distca_kv_shards *kv_shards, void *out_base, const int64_t *out_task_off,
+                                     int64_t out_tok_bytes, float *lse, const int32_t *cu_q, const int32_t *cu_k,
+                                     const int32_t *kv_off, const distca_ca_params *p, void *workspace, int64_t workspace_bytes,
+                                     void *stream) {
+  if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
+  if (!kv_shards) return fail(DISTCA_E_INVALID, "ca_fwd_buffers: null table of K/V shards");
+  return (p->dtype == DISTCA_DTYPE_F16 ? run_fwd_tokens_f16 : run_fwd_tokens)(q_base, q_task_off, q_tok_bytes, k, v, kv_shards, out_base,
+                                                                              out_task_off, out_tok_bytes, lse, cu_q, cu_k, kv_off, p,
+                                                                              workspace, workspace_bytes, stream);
+}
+
+namespace distca {
+int make_kv_shards(const distca_kv_shards *in, const int32_t *kv_off, bool backward, KvShards *out) {
+  if (in->num_shards <= 0) return fail(DISTCA_E_INVALID, "kv_shards: num_shards=%d", in->num_shards);
+  if (!in->row_start || !in->k_offset || !in->v_offset || !in->task_shard) return fail(DISTCA_E_INVALID, "kv_shards: null array");
+  if (backward && (!in->dk_offset || !in->dv_offset)) return fail(DISTCA_E_INVALID, "kv_shards: the backward needs dk_offset and dv_offset");
+  if (!kv_off) return fail(DISTCA_E_INVALID, "kv_shards: kv_task_offsets is required (tasks name stored rows)");
+  out->row_start = in->row_start; out->k_off = in->k_offset; out->v_off = in->v_offset;
+  out->dk_off = in->dk_offset; out->dv_off = in->dv_offset; out->task_shard = in->task_shard;
+  out->num_shards = in->num_shards;
+  return DISTCA_OK;
+}
+}  // namespace distca
 
 extern "C" int distca_ca_fwd(const void *q, const void *k, const void *v, void *out, float *lse, const int32_t *cu_q,
                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
@@ -499,9 +559,9 @@ extern "C" int distca_ca_fwd_noalloc(const void *q, const void *k, const void *v
 
 namespace distca {
 int DISTCA_FN(run_fwd_tokens)(const void *q_base, const int64_t *q_task_off, int64_t q_tok_bytes, const void *k, const void *v,
-                              void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes, float *lse, const int32_t *cu_q,
-                              const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p, void *workspace,
-                              int64_t workspace_bytes, void *stream) {
+                              const distca_kv_shards *kv_shards, void *out_base, const int64_t *out_task_off, int64_t out_tok_bytes,
+                              float *lse, const int32_t *cu_q, const int32_t *cu_k, const int32_t *kv_off, const distca_ca_params *p,
+                              void *workspace, int64_t workspace_bytes, void *stream) {
   const void *q = q_base;
   void *out = out_base;
   if (!p) return fail(DISTCA_E_INVALID, "ca_fwd: null params");
@@ -538,16 +598,25 @@ int DISTCA_FN(run_fwd_tokens)(const void *q_base, const int64_t *q_task_off, int
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   a.q_task_off = q_task_off; a.out_task_off = out_task_off; a.q_tok_bytes = q_tok_bytes; a.out_tok_bytes = out_tok_bytes;
   a.lse_in_token = lse ? 0 : 1;
+  a.shards = KvShards{};
+  if (kv_shards) {
+    rc = make_kv_shards(kv_shards, kv_off, false, &a.shards);
+    if (rc) return rc;
+  }
   const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
   if (device_setup_pending(kSlotFwdLds)) {
-    hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
+    hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
     if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
     device_setup_done(kSlotFwdLds);
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);
-    hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
+    if (kv_shards)
+      hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, true>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
+    else
+      hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, false>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
   }
   return check_launch("ca_fwd");
 }

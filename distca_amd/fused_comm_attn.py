@@ -287,15 +287,28 @@ class SharedKVOnDevice:
     num_rows: int
     k_grad_offset: Optional[Tensor] = None   # int64 [stored shards] into the send buffer (backward)
     v_grad_offset: Optional[Tensor] = None
+    row_start: Optional[Tensor] = None       # int32 [stored shards + 1]: first store row of every shard
+    task_shard: Optional[Tensor] = None      # int32 [tasks]: the stored shard that holds the first row of each task's prefix
 
     @classmethod
     def build(cls, layout, k_entry_offset: Tensor, v_entry_offset: Tensor, device, k_grad_entry_offset: Tensor = None,
               v_grad_entry_offset: Tensor = None) -> "SharedKVOnDevice":
         """`*_entry_offset`: host int64 tensors with one byte offset per K/V entry (aliases of a shard hold the same)."""
         pick = lambda t: None if t is None else t.cpu()[layout.entry_of_stored].to(device=device, dtype=torch.int64)
+        row_start = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(layout.store_tokens.cpu(), 0)])
+        task_shard = torch.searchsorted(row_start[1:].contiguous(), layout.kv_task_offsets.cpu().to(torch.int64), right=True)
+        task_shard = task_shard.clamp_max(max(len(layout.store_tokens) - 1, 0))
         return cls(layout.store_tokens.to(device), pick(k_entry_offset), pick(v_entry_offset),
                    layout.kv_task_offsets.to(device=device, dtype=torch.int32), layout.num_rows,
-                   pick(k_grad_entry_offset), pick(v_grad_entry_offset))
+                   pick(k_grad_entry_offset), pick(v_grad_entry_offset),
+                   row_start.to(device=device, dtype=torch.int32), task_shard.to(device=device, dtype=torch.int32))
+
+    def c_struct(self, backward: bool) -> "_lib.KvShards":
+        """struct distca_kv_shards over this layout's device arrays (which must outlive the call they are passed to)."""
+        ptr = lambda t: None if t is None else t.data_ptr()
+        return _lib.KvShards(int(self.store_tokens.numel()), ptr(self.row_start), ptr(self.k_offset), ptr(self.v_offset),
+                             ptr(self.task_shard), ptr(self.k_grad_offset) if backward else None,
+                             ptr(self.v_grad_offset) if backward else None)
 
 
 @dataclass
@@ -314,12 +327,15 @@ class ServerFwdMeta:
 
 
 def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdMeta, fa_params: PackedSeqParams,
-                      fa_args: FlashAttnArgs, dtype: torch.dtype = torch.bfloat16, in_place: bool = True):
+                      fa_args: FlashAttnArgs, dtype: torch.dtype = torch.bfloat16, in_place: bool = True,
+                      kv_shards_in_place: bool = True):
     """fused_comm_attn.py:298-389: unpack q,k,v -> attention -> pack [out | lse].
 
     With `in_place` (the default) the kernel reads the query tokens where they lie in the receive
-    buffer and writes the [out | lse] tokens where they belong in the send buffer; only K and V are
-    unpacked (a shard read by several tasks is copied once per task).  Returns (None, None) then.
+    buffer and writes the [out | lse] tokens where they belong in the send buffer.  With the one-copy
+    K/V layout (`meta.shared_kv`) it also reads the K/V shards where they lie (no pack kernel runs at
+    all; `kv_shards_in_place=False` unpacks every stored shard once instead); without that layout K and
+    V are unpacked as in the reference, a shard read by several tasks once per task.  Returns (None, None) then.
     Without it every step is its own pass, as in the reference, and (attn_out [T,Hq*D],
     softmax_lse [Hq,T]) are returned for the caller's own use.  Both leave the same bytes in the
     send buffer."""
@@ -327,12 +343,17 @@ def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdM
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
     in_place = in_place and dtype in _ELEM_CODE and d == HEAD_DIM
     shared = meta.shared_kv if in_place else None
+    # with the one-copy layout the kernel reads the K/V shards where they lie in the receive buffer: nothing is unpacked
+    kv_in_place = shared is not None and kv_shards_in_place and shared.row_start is not None and shared.num_rows > 0
     k_rows = shared.num_rows if shared is not None else meta.recv_k_shape[0]
-    recv_k = torch.empty((k_rows, meta.recv_k_shape[1]), dtype=dtype, device=dev)
-    recv_v = torch.empty_like(recv_k)
+    if not kv_in_place:
+        recv_k = torch.empty((k_rows, meta.recv_k_shape[1]), dtype=dtype, device=dev)
+        recv_v = torch.empty_like(recv_k)
     if in_place:
         kv_off = getattr(fa_params, "kv_task_offsets", None)
-        if shared is not None:
+        if kv_in_place:
+            kv_off = shared.kv_task_offsets
+        elif shared is not None:
             # one copy of every K/V shard, documents contiguous: every task reads its prefix in place
             a2a_memcpy_non_cp_multi([recv_k, recv_v], [shared.k_offset, shared.v_offset], [shared.store_tokens] * 2, False,
                                     buffer=recv_buffer)
@@ -357,11 +378,19 @@ def ca_server_forward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerFwdM
             if t.dtype != torch.int64 or not t.is_cuda or t.numel() != cu_q.shape[0] - 1:
                 raise RuntimeError(f"{name} must be an int64 CUDA tensor with one entry per task")
         with torch.cuda.device(dev):
-            rc = lib.distca_ca_fwd_tokens(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), q_tok, recv_k.data_ptr(),
-                                          recv_v.data_ptr(), send_buffer.data_ptr(), meta.out_send_offset.data_ptr(), out_tok,
-                                          None, cu_q.data_ptr(), cu_k.data_ptr(), kv_off.data_ptr() if kv_off is not None else None,
-                                          ctypes.byref(p), ws.data_ptr(),
-                                          ws.numel(), torch.cuda.current_stream().cuda_stream)
+            if kv_in_place:
+                shards = shared.c_struct(False)
+                rc = lib.distca_ca_fwd_buffers(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), q_tok, recv_buffer.data_ptr(),
+                                               recv_buffer.data_ptr(), ctypes.byref(shards), send_buffer.data_ptr(),
+                                               meta.out_send_offset.data_ptr(), out_tok, None, cu_q.data_ptr(), cu_k.data_ptr(),
+                                               kv_off.data_ptr(), ctypes.byref(p), ws.data_ptr(), ws.numel(),
+                                               torch.cuda.current_stream().cuda_stream)
+            else:
+                rc = lib.distca_ca_fwd_tokens(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), q_tok, recv_k.data_ptr(),
+                                              recv_v.data_ptr(), send_buffer.data_ptr(), meta.out_send_offset.data_ptr(), out_tok,
+                                              None, cu_q.data_ptr(), cu_k.data_ptr(), kv_off.data_ptr() if kv_off is not None else None,
+                                              ctypes.byref(p), ws.data_ptr(),
+                                              ws.numel(), torch.cuda.current_stream().cuda_stream)
         _lib.check(rc, "ca_server_forward")
         return None, None
     recv_q = torch.empty(meta.recv_q_shape, dtype=dtype, device=dev)
@@ -396,7 +425,7 @@ class ServerBwdMeta:
 
 def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwdMeta, fa_args: FlashAttnArgs,
                        cu_seqlens_q: Tensor, cu_seqlens_kv: Tensor, max_seqlen_q: int, max_seqlen_kv: int,
-                       dtype: torch.dtype = torch.bfloat16, in_place: bool = True):
+                       dtype: torch.dtype = torch.bfloat16, in_place: bool = True, kv_shards_in_place: bool = True):
     """fused_comm_attn.py:407-461: unpack merged request -> attention backward -> sum
     duplicate KV gradients -> masked pack of dq, dk, dv.
 
@@ -404,8 +433,11 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
     aligned) the kernels read dO, O, lse and q where they lie in the receive buffer and write dq
     where it belongs in the send buffer; K and V are unpacked (with `meta.shared_kv` every stored shard once, and
     dk / dv then come out summed over the tasks that read a shard and are packed once), dk and dv otherwise summed
-    over the duplicate copies and packed as before.  Returns (None, dk, dv) then, else (dq, dk, dv).  Both leave the same bytes in the send
-    buffer."""
+With that layout and `kv_shards_in_place` (the default) the kernels also read the K/V shards where they lie
+    and write the shards' dk / dv where they belong in the send buffer: no pack kernel runs, and (None, None, None)
+    is returned.  Otherwise returns (None, dk, dv) when in place, else (dq, dk, dv).  dq bytes in the send buffer are
+    the same in every form; dk / dv of the one-copy forms are summed in fp32 and rounded once, those of the step-by-step
+    form are bf16 sums of per-task bf16 gradients, as in the reference."""
     dev = recv_buffer.device
     hq, hkv, d = fa_args.num_heads_q, fa_args.num_heads_kv, fa_args.head_dim
     in_place = in_place and (hq * 4) % 16 == 0 and dtype in _ELEM_CODE and d == HEAD_DIM
@@ -413,6 +445,34 @@ def ca_server_backward(recv_buffer: Tensor, send_buffer: Tensor, meta: ServerBwd
     # sums dK/dV over the document's tasks in registers
     shared = meta.shared_kv if in_place else None
     k_rows = shared.num_rows if shared is not None else meta.k_shape[0]
+    kv_in_place = (shared is not None and kv_shards_in_place and shared.row_start is not None and shared.num_rows > 0
+                   and shared.k_grad_offset is not None and int(cu_seqlens_q.shape[0]) > 1 and int(meta.attn_out_shape[0]) > 0)
+    if kv_in_place:
+        # everything where it lies: request tokens and K/V shards read from the receive buffer, dq tokens and the
+        # shards' dk / dv written into the send buffer; no pack kernel runs
+        tq = int(meta.attn_out_shape[0])
+        scale = fa_args.softmax_scale if fa_args.softmax_scale is not None else d ** (-0.5)
+        lib = _lib.load()
+        p = _params(cu_seqlens_q.shape[0] - 1, tq, int(k_rows), hq, hkv, d, max_seqlen_q, max_seqlen_kv, scale, fa_args.causal,
+                    fa_args.deterministic, dtype)
+        need = lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))
+        if need < 0:
+            _lib.check(int(need), "ca_server_backward")
+        ws = _workspace(None, int(need), dev)
+        row = hq * d * 2
+        req_tok = size_pad_by_int4(3 * row + hq * 4, 1)[0]
+        for name, t in (("q_recv_offset", meta.q_recv_offset), ("q_grad_send_offset", meta.q_grad_send_offset)):
+            if t.dtype != torch.int64 or not t.is_cuda or t.numel() != cu_seqlens_q.shape[0] - 1:
+                raise RuntimeError(f"{name} must be an int64 CUDA tensor with one entry per task")
+        shards = shared.c_struct(True)
+        with torch.cuda.device(dev):
+            rc = lib.distca_ca_bwd_buffers(recv_buffer.data_ptr(), meta.q_recv_offset.data_ptr(), req_tok, recv_buffer.data_ptr(),
+                                           recv_buffer.data_ptr(), ctypes.byref(shards), send_buffer.data_ptr(),
+                                           meta.q_grad_send_offset.data_ptr(), row, send_buffer.data_ptr(), send_buffer.data_ptr(),
+                                           cu_seqlens_q.data_ptr(), cu_seqlens_kv.data_ptr(), shared.kv_task_offsets.data_ptr(),
+                                           ctypes.byref(p), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "ca_server_backward")
+        return None, None, None
     recv_k = torch.empty((k_rows, meta.k_shape[1]), dtype=dtype, device=dev)
     recv_v = torch.empty_like(recv_k)
     if in_place:

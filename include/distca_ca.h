@@ -223,6 +223,35 @@ int distca_ca_fwd_tokens(const void *q_base, const int64_t *q_task_off,
                          const distca_ca_params *p, void *workspace,
                          int64_t workspace_bytes, void *stream);
 
+/* The same forward with K and V, too, read where the CA server has them: every stored
+ * K/V shard lies once somewhere in the receive buffer, and instead of unpacking the
+ * shards into contiguous tensors first (post_a2a_qkv,
+ * distca/runtime/attn_kernels/dispatch.py:60-94) the kernel addresses a stored row
+ * through the table of shards.  Stored rows [row_start[s], row_start[s+1]) are the rows
+ * of shard s and lie token after token (Hkv*D elements each) from byte k_offset[s] of
+ * `k` (v_offset[s] of `v`; both may be the same buffer).  kv_task_offsets (required)
+ * names stored rows, p->total_k = row_start[num_shards], and task_shard[b] is the shard
+ * that holds row kv_task_offsets[b].  Offsets are multiples of 16.  All arrays are
+ * device arrays; the ranges they name are the caller's responsibility. */
+typedef struct distca_kv_shards {
+  int32_t num_shards;
+  const int32_t *row_start;  /* int32 [num_shards + 1], ascending                  */
+  const int64_t *k_offset;   /* int64 [num_shards]                                 */
+  const int64_t *v_offset;   /* int64 [num_shards]                                 */
+  const int32_t *task_shard; /* int32 [num_tasks]                                  */
+  const int64_t *dk_offset;  /* backward only: where the shards' dK / dV rows go,  */
+  const int64_t *dv_offset;  /* byte offsets from `dk` / `dv`                      */
+} distca_kv_shards;
+int distca_ca_fwd_buffers(const void *q_base, const int64_t *q_task_off,
+                          int64_t q_tok_bytes, const void *k, const void *v,
+                          const distca_kv_shards *kv_shards, void *out_base,
+                          const int64_t *out_task_off, int64_t out_tok_bytes,
+                          float *lse, const int32_t *cu_seqlens_q,
+                          const int32_t *cu_seqlens_k,
+                          const int32_t *kv_task_offsets,
+                          const distca_ca_params *p, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+
 /* dk/dv rows are written once per task when kv_task_offsets is NULL.  When it
  * is given, dk/dv of a stored row hold the sum over every task that read the
  * row (what the reference obtains with duplicated KV copies and
@@ -257,6 +286,23 @@ int distca_ca_bwd_tokens(const void *req_base, const int64_t *req_task_off,
                          const int32_t *kv_task_offsets,
                          const distca_ca_params *p, void *workspace,
                          int64_t workspace_bytes, void *stream);
+
+/* The backward with K and V read through the table of shards as in
+ * distca_ca_fwd_buffers, and dK / dV written where the shards' gradients belong in the
+ * send buffer (dk_offset[s] / dv_offset[s] from `dk` / `dv`) instead of into
+ * contiguous tensors that a pack pass would copy there (pre_a2a_qkv in backward,
+ * attn_kernels/dispatch.py:39-56).  Every stored row is written: rows no task reads
+ * as zeros.  Key blocks are never cut into pieces in this form (no float atomics:
+ * the result is the same in every run). */
+int distca_ca_bwd_buffers(const void *req_base, const int64_t *req_task_off,
+                          int64_t req_tok_bytes, const void *k, const void *v,
+                          const distca_kv_shards *kv_shards, void *dq_base,
+                          const int64_t *dq_task_off, int64_t dq_tok_bytes,
+                          void *dk, void *dv, const int32_t *cu_seqlens_q,
+                          const int32_t *cu_seqlens_k,
+                          const int32_t *kv_task_offsets,
+                          const distca_ca_params *p, void *workspace,
+                          int64_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Tile scheduler, host mirror.  The device builds the same list inside

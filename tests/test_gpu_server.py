@@ -605,3 +605,108 @@ def test_fused_comm_attn_autograd_function(cuda):
     assert r0.data_ptr() == DispatcherWrapper.instance[0].recv_buffer.data_ptr()
     assert s1.data_ptr() == DispatcherWrapper.instance[1].send_buffer.data_ptr() and DispatcherWrapper.cur_instance == 1
     DispatcherWrapper.instance = None
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4)])
+def test_kv_shards_read_in_place_equal_dense_tensors(cuda, hq, hkv):
+    """distca_ca_fwd_buffers / distca_ca_bwd_buffers with K/V shards of odd lengths (1 to 300 rows: tiles of 32 and 64
+    keys and key blocks of 256 straddle them every which way) scattered through a buffer in shuffled order, K and V in
+    separate places, with unused bytes between them: out, lse, dq, and dk / dv gathered back from the shards' places in
+    the gradient buffer, are bit for bit what the entry points over dense tensors with kv_task_offsets give
+    (deterministic backward; the arithmetic is the same, only the addresses differ), rows that no task reads come back
+    as zeros, and nothing outside the shards' places is written."""
+    import ctypes
+    from distca_amd import _lib
+    from distca_amd.fused_comm_attn import _params, ca_varlen_bwd, ca_varlen_fwd
+    rng = np.random.default_rng(hq)
+    d = 128
+    # three stored documents; tasks are prefixes of them (the second document is only read up to row 500 of 650)
+    doc_rows = [700, 650, 130]
+    doc_start = np.concatenate([[0], np.cumsum(doc_rows)])
+    total_k = int(doc_start[-1])
+    task_doc = [0, 0, 0, 1, 1, 2, 0]
+    k_lens = np.array([255, 257, 700, 33, 500, 130, 700], dtype=np.int64)
+    q_lens = np.array([255, 2, 443, 33, 212, 64, 100], dtype=np.int64)
+    kv_off = np.array([doc_start[t] for t in task_doc], dtype=np.int32)
+    # shards: every document cut at random places
+    shard_len = []
+    for n in doc_rows:
+        left = n
+        while left > 0:
+            c = int(min(left, rng.integers(1, 301)))
+            shard_len.append(c); left -= c
+    shard_len = np.array(shard_len, dtype=np.int64)
+    ns = len(shard_len)
+    row_start = np.concatenate([[0], np.cumsum(shard_len)]).astype(np.int32)
+    task_shard = (np.searchsorted(row_start[1:], kv_off, side="right")).astype(np.int32)
+    rb = hkv * d * 2
+    def scatter_offsets(seed, base):
+        order = np.random.default_rng(seed).permutation(ns)
+        off = np.zeros(ns, dtype=np.int64)
+        cur = base
+        for s_ in order:
+            off[s_] = cur
+            cur += int(shard_len[s_]) * rb + 16 * int(np.random.default_rng(seed + s_).integers(0, 5))   # a gap of 0..64 bytes
+        return off, cur
+    k_offs, end_k = scatter_offsets(1, 48)
+    v_offs, end_v = scatter_offsets(2, end_k + 32)
+    dk_offs, end_dk = scatter_offsets(3, 16)
+    dv_offs, end_dv = scatter_offsets(4, end_dk)
+    tq = int(q_lens.sum())
+    q, k, v, do = (t.to(cuda) for t in make_qkv(tq, total_k, hq, hkv, d, 77))
+    kvbuf = torch.full((end_v + 64,), 0x7F, dtype=torch.uint8, device=cuda)       # 0x7f7f as bf16 is a NaN: a stray read shows
+    kb_, vb_ = k.reshape(total_k, -1).view(torch.uint8), v.reshape(total_k, -1).view(torch.uint8)
+    for s_ in range(ns):
+        r0, r1 = int(row_start[s_]), int(row_start[s_ + 1])
+        kvbuf[k_offs[s_]:k_offs[s_] + (r1 - r0) * rb] = kb_[r0:r1].reshape(-1)
+        kvbuf[v_offs[s_]:v_offs[s_] + (r1 - r0) * rb] = vb_[r0:r1].reshape(-1)
+    i32 = lambda x: torch.tensor(np.asarray(x), dtype=torch.int32, device=cuda)
+    i64 = lambda x: torch.tensor(np.asarray(x), dtype=torch.int64, device=cuda)
+    cu_q, cu_k, off_d = i32(np.concatenate([[0], np.cumsum(q_lens)])), i32(np.concatenate([[0], np.cumsum(k_lens)])), i32(kv_off)
+    mq, mk = int(q_lens.max()), int(k_lens.max())
+    out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, kv_task_offsets=off_d)
+    dq, dk, dv = ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, deterministic=True, kv_task_offsets=off_d)
+
+    lib = _lib.load()
+    dev_arrays = dict(row_start=i32(row_start), k=i64(k_offs), v=i64(v_offs), ts=i32(task_shard), dk=i64(dk_offs), dv=i64(dv_offs))
+    shards = _lib.KvShards(ns, dev_arrays["row_start"].data_ptr(), dev_arrays["k"].data_ptr(), dev_arrays["v"].data_ptr(),
+                           dev_arrays["ts"].data_ptr(), dev_arrays["dk"].data_ptr(), dev_arrays["dv"].data_ptr())
+    p = _params(len(q_lens), tq, total_k, hq, hkv, d, mq, mk, d ** -0.5, True, True)
+    ws = torch.empty((int(lib.distca_ca_bwd_workspace_bytes(ctypes.byref(p))),), dtype=torch.uint8, device=cuda)
+    stream = torch.cuda.current_stream().cuda_stream
+    print("forward over shards in place", flush=True)
+    out2, lse2 = torch.empty_like(out), torch.empty_like(lse)
+    _lib.check(lib.distca_ca_fwd_buffers(q.data_ptr(), None, 0, kvbuf.data_ptr(), kvbuf.data_ptr(), ctypes.byref(shards), out2.data_ptr(),
+                                         None, 0, lse2.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(), off_d.data_ptr(), ctypes.byref(p),
+                                         ws.data_ptr(), ws.numel(), stream), "fwd_buffers")
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+    # request tokens [dO | O | lse | q], one region per task in task order
+    row = hq * d * 2
+    req_tb = 3 * row + hq * 4
+    req = torch.empty((tq, req_tb), dtype=torch.uint8, device=cuda)
+    for c0, part in ((0, do.reshape(tq, -1)), (row, out.reshape(tq, -1)), (2 * row, lse.T.contiguous()), (2 * row + hq * 4, q.reshape(tq, -1))):
+        pb_ = part.contiguous().view(torch.uint8).view(tq, -1)
+        req[:, c0:c0 + pb_.shape[1]] = pb_
+    tok_off = np.concatenate([[0], np.cumsum(q_lens)[:-1]])
+    req_off, dq_off = i64(tok_off * req_tb), i64(tok_off * row)
+    dq2 = torch.empty_like(dq)
+    gbuf = torch.full((end_dv + 64,), 0x3C, dtype=torch.uint8, device=cuda)
+    print("backward over shards in place", flush=True)
+    _lib.check(lib.distca_ca_bwd_buffers(req.data_ptr(), req_off.data_ptr(), req_tb, kvbuf.data_ptr(), kvbuf.data_ptr(), ctypes.byref(shards),
+                                         dq2.data_ptr(), dq_off.data_ptr(), row, gbuf.data_ptr(), gbuf.data_ptr(), cu_q.data_ptr(),
+                                         cu_k.data_ptr(), off_d.data_ptr(), ctypes.byref(p), ws.data_ptr(), ws.numel(), stream), "bwd_buffers")
+    torch.cuda.synchronize()
+    assert torch.equal(dq2, dq)
+    g = gbuf.cpu()
+    touched = torch.zeros(g.numel(), dtype=torch.bool)
+    for name, offs, dense in (("dk", dk_offs, dk), ("dv", dv_offs, dv)):
+        dense_b = dense.reshape(total_k, -1).view(torch.uint8).cpu()
+        for s_ in range(ns):
+            r0, r1 = int(row_start[s_]), int(row_start[s_ + 1])
+            got = g[offs[s_]:offs[s_] + (r1 - r0) * rb].reshape(r1 - r0, rb)
+            assert torch.equal(got, dense_b[r0:r1]), f"{name} of shard {s_} (stored rows {r0}..{r1})"
+            touched[offs[s_]:offs[s_] + (r1 - r0) * rb] = True
+    assert (g[~touched] == 0x3C).all(), "bytes outside the shards' places were written"
+    # rows 500..650 of the second document are read by no task: zeros in the dense result, hence in the shards
+    assert (dk[int(doc_start[1]) + 500:int(doc_start[2])] == 0).all() and (dv[int(doc_start[1]) + 500:int(doc_start[2])] == 0).all()
