@@ -254,6 +254,94 @@ def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap:
     return res
 
 
+def mfma_probe(torch, _lib, dev, executed_tflops: float, rounds: int = 5, warm_seconds: float = 0.6):
+    """What this device delivers for the MFMA instruction itself, measured right after the attention steps: a loop of
+    MFMAs on every SIMD, alone and with other work in every MFMA's shadow.  The shader clock under such a load takes a
+    few hundred milliseconds to settle at what the power limit allows, so the MFMA-only loop first runs for
+    `warm_seconds`; the four variants are then run interleaved, round after round, and the median and the spread over
+    the rounds are reported per variant (so that a clock still drifting cannot favour whichever variant runs last)."""
+    scratch = torch.zeros(4, dtype=torch.int64, device=dev)
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+    kinds = (("mfma_only", _lib.PROBE_MFMA_ONLY), ("with_1kb_lds_read_per_mfma", _lib.PROBE_LDS_READ),
+             ("with_4_fma_per_mfma", _lib.PROBE_FMA4), ("with_2_exp_per_mfma", _lib.PROBE_EXP2))
+    iters = 20000
+    for _, kind in kinds:    # the first launch of a kernel also loads it
+        _lib.probe_mfma_rate(kind, 200, scratch.data_ptr(), stream_ptr)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < warm_seconds:
+        _lib.probe_mfma_rate(_lib.PROBE_MFMA_ONLY, iters, scratch.data_ptr(), stream_ptr)
+    runs = {name: [] for name, _ in kinds}
+    for _ in range(rounds):
+        for name, kind in kinds:
+            runs[name].append(_lib.probe_mfma_rate(kind, iters, scratch.data_ptr(), stream_ptr))
+    probe = {"rounds": rounds}
+    for name, _ in kinds:
+        tf = sorted(r[0] for r in runs[name])
+        probe[name] = {"TFLOP/s": round(float(np.median(tf)), 1), "TFLOP/s_min": round(tf[0], 1), "TFLOP/s_max": round(tf[-1], 1),
+                       "cycles_per_mfma": round(float(np.median([r[1] for r in runs[name]])), 2),
+                       "clock_GHz": round(float(np.median([r[2] for r in runs[name]])), 3)}
+    probe["executed_TFLOP/s_of_the_three_attention_kernels"] = round(executed_tflops, 1)
+    probe["executed_over_mfma_only"] = round(executed_tflops / probe["mfma_only"]["TFLOP/s"], 4)
+    probe["note"] = (f"v_mfma_f32_32x32x16_bf16 on pseudo-random operands, one wave per SIMD on every SIMD, {8 * iters} per wave and run; "
+                     f"{warm_seconds} s of the MFMA-only loop first, then the four variants interleaved for {rounds} rounds: median (min..max) "
+                     "rate by HIP events, clock by the device's cycle and real-time counters: what the power limit leaves "
+                     "of the published 2.5 PFLOP/s (every pipe busy at 2.4 GHz) on this device for this instruction")
+    return probe
+
+
+def other_workloads_bench(torch, dev, steps: int = 2):
+    """The other attention configurations and two batches of short CA tasks through the same entry points: kernel times by
+    the library's events (no gaps between launches), algorithmic TFLOP/s.  Parity of these configurations is the
+    test suite's business (tests/test_gpu_scale.py); this leg times them where the headline is timed."""
+    from distca_amd import _lib
+    from distca_amd.fused_comm_attn import ca_varlen_bwd, ca_varlen_fwd
+    from distca_amd import workloads
+    short = np.full(128, 1024, dtype=np.int64)
+    cases = [
+        ("cfg3b_ca_tasks", workloads.config3_ca_tasks(variant="b"), "15 CA tasks over shared K/V prefixes of up to 524288 rows, 262144 query rows, 32q/8kv, deterministic"),
+        ("cfg5_llama70b_skewed", workloads.config5_llama70b_skewed(), "524288 tokens with one 262144-token document, 64q/8kv"),
+        ("short_documents", workloads.TaskBatch("128x1024", short, short.copy(), 32, 8), "128 whole documents of 1024 tokens, 32q/8kv"),
+        ("shards_4096_long_prefixes", workloads.config3_ca_tasks(variant="a", total_q=131072, num_docs=4, max_doc=131072, seed=5013),
+         "32 CA tasks of 4096 query rows over shared K/V prefixes of up to 131072 rows, 32q/8kv, deterministic"),
+    ]
+    res = {}
+    for name, b, what in cases:
+        hq, hkv, d = b.num_heads_q, b.num_heads_kv, b.head_dim
+        gen = torch.Generator(device=dev).manual_seed(7)
+        rnd = lambda *shape: torch.randn(shape, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        q, k, v, do = rnd(b.total_q, hq, d), rnd(b.kv_rows, hkv, d), rnd(b.kv_rows, hkv, d), rnd(b.total_q, hq, d)
+        cu_q, cu_k = torch.from_numpy(b.cu_seqlens_q).to(dev), torch.from_numpy(b.cu_seqlens_k).to(dev)
+        off = torch.tensor(b.kv_task_offsets, dtype=torch.int32, device=dev) if b.kv_task_offsets is not None else None
+        mq, mk = int(b.q_lens.max()), int(b.k_lens.max())
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+        def step():
+            out, lse = ca_varlen_fwd(q, k, v, cu_q, cu_k, mq, mk, None, True, off)
+            ca_varlen_bwd(do, q, k, v, out, lse, cu_q, cu_k, mq, mk, None, True, off is not None, off, dq, dk, dv)
+
+        step()
+        torch.cuda.synchronize()
+        timers = (_lib.TIMER_CA_FWD, _lib.TIMER_CA_BWD_DQ, _lib.TIMER_CA_BWD)
+        for t in timers:
+            _lib.timing_read(t)
+        _lib.timing_enable(True)
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        _lib.timing_enable(False)
+        fwd, dqk, dkdv = (_lib.timing_read(t)[0] / steps for t in timers)
+        f_fwd, f_bwd = b.flops()
+        tf = lambda flop, ms: round(flop / (ms * 1e-3) / 1e12, 1)
+        res[name] = {"workload": what, "causal_pairs": b.causal_pairs, "steps": steps,
+                     "ca_fwd_kernel_ms": round(fwd, 3), "ca_bwd_dq64_kernel_ms": round(dqk, 3), "ca_bwd_dkdv64_kernel_ms": round(dkdv, 3),
+                     "fwd_TFLOP/s": tf(f_fwd, fwd), "bwd_TFLOP/s": tf(f_bwd, dqk + dkdv), "fwd_bwd_TFLOP/s": tf(f_fwd + f_bwd, fwd + dqk + dkdv),
+                     "pct_of_bf16_mfma_peak": round(100 * (f_fwd + f_bwd) / ((fwd + dqk + dkdv) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2)}
+        log(f"  {name:26s} fwd {fwd:9.3f} ms ({res[name]['fwd_TFLOP/s']} TFLOP/s)  bwd {dqk:.3f} + {dkdv:.3f} ms ({res[name]['bwd_TFLOP/s']})  "
+            f"fwd+bwd {res[name]['fwd_bwd_TFLOP/s']} TFLOP/s = {res[name]['pct_of_bf16_mfma_peak']} %")
+        del q, k, v, do, dq, dk, dv
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -264,6 +352,7 @@ def main():
     ap.add_argument("--no-pack", action="store_true")
     ap.add_argument("--no-tick", action="store_true")
     ap.add_argument("--no-probe", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other attention configurations (cfg3b, cfg5, short tasks)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the CA-server path; --gpus must be 1 "
@@ -331,21 +420,10 @@ def main():
     # a loop of MFMAs on every SIMD, alone and with other work in every MFMA's shadow
     probe = None
     if not args.no_probe:
-        scratch = torch.zeros(4, dtype=torch.int64, device=dev)
-        stream_ptr = torch.cuda.current_stream().cuda_stream
-        probe = {}
-        for name, kind in (("mfma_only", _lib.PROBE_MFMA_ONLY), ("with_1kb_lds_read_per_mfma", _lib.PROBE_LDS_READ),
-                           ("with_4_fma_per_mfma", _lib.PROBE_FMA4), ("with_2_exp_per_mfma", _lib.PROBE_EXP2)):
-            for _ in range(3):  # the last of three runs: the clock has settled by then
-                tf, cyc, ghz = _lib.probe_mfma_rate(kind, 20000, scratch.data_ptr(), stream_ptr)
-            probe[name] = {"TFLOP/s": round(tf, 1), "cycles_per_mfma": round(cyc, 2), "clock_GHz": round(ghz, 3)}
         executed = 1e-12 * (flop_fwd + 1.4 * flop_bwd) / ((fwd_k + bwd_k) * 1e-3)  # S and dP are computed in both backward kernels
-        probe["executed_TFLOP/s_of_the_three_attention_kernels"] = round(executed, 1)
-        probe["executed_over_mfma_only"] = round(executed / probe["mfma_only"]["TFLOP/s"], 4)
-        probe["note"] = ("v_mfma_f32_32x32x16_bf16 on pseudo-random operands, one wave per SIMD on every SIMD, 160000 per wave; "
-                         "rate by HIP events, clock by the device's cycle and real-time counters: what the power limit leaves "
-                         "of the published 2.5 PFLOP/s (every pipe busy at 2.4 GHz) on this device for this instruction")
-        log(f"  MFMA-only loop {probe['mfma_only']['TFLOP/s']} TFLOP/s at {probe['mfma_only']['clock_GHz']} GHz; the attention kernels execute "
+        probe = mfma_probe(torch, _lib, dev, executed)
+        log(f"  MFMA-only loop {probe['mfma_only']['TFLOP/s']} TFLOP/s (median of {probe['rounds']} rounds, {probe['mfma_only']['TFLOP/s_min']}"
+            f"..{probe['mfma_only']['TFLOP/s_max']}) at {probe['mfma_only']['clock_GHz']} GHz; the attention kernels execute "
             f"{probe['executed_TFLOP/s_of_the_three_attention_kernels']} TFLOP/s = {100 * probe['executed_over_mfma_only']:.1f} % of it")
 
     pack = None
@@ -365,6 +443,12 @@ def main():
             f"K/V unpacked first: {tick['forward_kv_unpacked_ms']}, kernel {tick['forward_kv_unpacked_attention_kernel_ms']}), "
             f"backward {tick['backward_ms']} ms (kernels {tick['backward_attention_kernels_ms']}; K/V unpacked first: "
             f"{tick['backward_kv_unpacked_ms']}, kernels {tick['backward_kv_unpacked_attention_kernels_ms']})")
+
+    extra = None
+    if not args.no_extra:
+        del q, k, v, do
+        torch.cuda.empty_cache()
+        extra = other_workloads_bench(torch, dev)
 
     cpu = None
     if args.cpu_seconds > 0:
@@ -393,6 +477,7 @@ def main():
         "cpu_baseline": cpu,
         "pack_unpack": pack,
         "server_tick": tick,
+        "extra": extra,
     }
     print(json.dumps(line), flush=True)
 
