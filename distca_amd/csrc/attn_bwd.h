@@ -28,6 +28,7 @@ struct BwdArgs {
   int32_t *tickets;  // one counter per kv head (sched.h)
   const void *zero_row;  // 256 zero bytes: source of tile rows past the end of a task
   int32_t sched_items_off;
+  int32_t merge_tiles;  // dQ kernel: merge_tiles of its list (sched.h, fwd_merge), 0 = one block per item
   int32_t hq, hkv, group, total_q;
   uint32_t group_magic;  // ceil(2^32 / group), 0 when group == 1: n / group == umulhi(n, magic) for n * group < 2^32
   int32_t causal;

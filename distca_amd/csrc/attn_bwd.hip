@@ -266,6 +266,7 @@ int DISTCA_FN(run_bwd)(const BwdQuerySide &qs, const void *k, const void *v, voi
   // statistics (lse in the log2 domain, -delta) in the workspace, which the dK/dV kernel reads.
   {
     const SchedGeom geom = dq_geom(p);
+    a.merge_tiles = geom.merge_tiles;
     const int64_t max_items = dq_max_items(p);
     rc = launch_build_schedule(0, cu_q, cu_k, p->num_tasks, geom, (int32_t *)(ws + w.sched_q), max_items, s);
     if (rc) return rc;

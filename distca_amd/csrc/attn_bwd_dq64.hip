@@ -70,14 +70,16 @@ __device__ __forceinline__ void mfma32_va0(f32x16 &acc, elemx8 a, accop_t b) {
 }
 
 // SEG: K/V rows are addressed through a table of shards (kv_shards.h) instead of as one dense tensor.
-template <bool SEG>
+// MERGE: a work item is several consecutive blocks of a task's query rows (sched.h, fwd_merge), worked off one after the
+// other; otherwise it is one block.
+template <bool SEG, bool MERGE>
 __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   int item, kvh;
   if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
   const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
-  const int task = it4.x, mblk = it4.y;
+  const int task = it4.x;
 
   const int q0 = a.cu_q[task];
   const int64_t qs_task = a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes;
@@ -88,11 +90,28 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   const int G = a.group;
   const int shift = lk - lq;
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int nrows = lq * G;
+  // the blocks of this item
+  int mb_first = it4.y, mb_end = it4.y + 1;
+  if constexpr (MERGE) {
+    SchedGeom geom;
+    geom.rows_per_block = kRowsWg; geom.kv_per_block = kFwdKV; geom.group = G; geom.causal = a.causal; geom.merge_tiles = a.merge_tiles;
+    const int m = fwd_merge(geom, lq, lk), nblk = (nrows + kRowsWg - 1) / kRowsWg;
+    mb_first = it4.y * m;
+    mb_end = mb_first + m < nblk ? mb_first + m : nblk;
+  }
+  // (a jump back rather than a loop statement: without MERGE the body below is then straight-line code, exactly the
+  // kernel that takes one block per item)
+  int mblk = mb_first;
+next_block:
+  // MERGE: the thread index is made opaque once per block, so that what derives from it is computed afresh for every
+  // block instead of being carried, and partly spilled, across the whole body
+  int tid_ = threadIdx.x;
+  if constexpr (MERGE) asm volatile("" : "+v"(tid_));
+  const int tid = tid_, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5;
   const int row_wg = mblk * kRowsWg;
-  const int nrows = lq * G;
 
   int tok_end = (row_wg + kRowsWg + G - 1) / G;
   if (tok_end > lq) tok_end = lq;
@@ -440,21 +459,32 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
         }
     }
   }
+  if constexpr (MERGE) {
+    if (++mblk < mb_end) {
+      __syncthreads();  // every wave has left the ring's stages before the next block's first tiles are requested
+      goto next_block;
+    }
+  }
 }
 
 }  // namespace
 
 int DISTCA_FN(launch_dq64)(const BwdArgs &a, int64_t grid, hipStream_t stream) {
   if (device_setup_pending(kSlotBwdDq64)) {
-    hipError_t e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ca_bwd_dq64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS: %s", kLds, hipGetErrorString(e));
+    const void *kernels[] = {(const void *)ca_bwd_dq64_kernel<false, false>, (const void *)ca_bwd_dq64_kernel<true, false>,
+                             (const void *)ca_bwd_dq64_kernel<false, true>, (const void *)ca_bwd_dq64_kernel<true, true>};
+    for (const void *kf : kernels) {
+      hipError_t e = hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+      if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_bwd: cannot reserve %d B of LDS: %s", kLds, hipGetErrorString(e));
+    }
     device_setup_done(kSlotBwdDq64);
   }
-  if (a.shards.num_shards > 0)
-    hipLaunchKernelGGL(ca_bwd_dq64_kernel<true>, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
-  else
-    hipLaunchKernelGGL(ca_bwd_dq64_kernel<false>, dim3((unsigned)grid), dim3(kThreads), kLds, stream, a);
+  const dim3 g((unsigned)grid), b(kThreads);
+  const bool seg = a.shards.num_shards > 0, merge = a.merge_tiles > 0;
+  if (seg && merge) hipLaunchKernelGGL((ca_bwd_dq64_kernel<true, true>), g, b, kLds, stream, a);
+  else if (seg) hipLaunchKernelGGL((ca_bwd_dq64_kernel<true, false>), g, b, kLds, stream, a);
+  else if (merge) hipLaunchKernelGGL((ca_bwd_dq64_kernel<false, true>), g, b, kLds, stream, a);
+  else hipLaunchKernelGGL((ca_bwd_dq64_kernel<false, false>), g, b, kLds, stream, a);
   return DISTCA_OK;
 }
 

@@ -45,15 +45,32 @@ inline int validate_params(const distca_ca_params *p) {
   return DISTCA_OK;
 }
 
+// Batches of short tasks have the forward and dQ kernels work off several consecutive blocks of a task per work item
+// (sched.h, fwd_merge).  Whether a batch is one is decided from host-known sizes, the mean task length: the kernels
+// built for merged items carry a loop around their body, which the ones for long tasks are spared.
+constexpr int32_t kMergeMeanTokens = 2048;  // batches whose tasks average fewer query tokens than this
+#ifndef DISTCA_MERGE_TILES_FWD
+#define DISTCA_MERGE_TILES_FWD 128
+#endif
+constexpr int32_t kMergeTilesFwd = DISTCA_MERGE_TILES_FWD;  // KV tiles (of 64 keys) a merged forward item aims for
+#ifndef DISTCA_MERGE_TILES_DQ
+#define DISTCA_MERGE_TILES_DQ 128
+#endif
+constexpr int32_t kMergeTilesDq = DISTCA_MERGE_TILES_DQ;    // the same for a merged dQ item (its list counts keys in the same unit)
+inline bool merge_short_tasks(const distca_ca_params *p) {
+  return p->num_tasks > 0 && (int64_t)p->total_q < (int64_t)kMergeMeanTokens * p->num_tasks;
+}
 inline SchedGeom fwd_geom(const distca_ca_params *p) {
   SchedGeom g;
   g.split_target = 0;
   g.walk_round = 0;
+  g.merge_tiles = merge_short_tasks(p) ? kMergeTilesFwd : 0;
   g.rows_per_block = kFwdRows;
   g.kv_per_block = kFwdKV;
   g.group = p->num_heads_q / p->num_heads_kv;
   g.causal = p->causal != 0;
-  g.cost_shift = pick_cost_shift((int64_t)p->max_seqlen_k / kFwdKV + 1);
+  const int64_t worst = (int64_t)p->max_seqlen_k / kFwdKV + 1;
+  g.cost_shift = pick_cost_shift(worst > g.merge_tiles ? worst : g.merge_tiles);
   return g;
 }
 // Key blocks are cut into pieces (sched.h) when the batch has so few of them that they could not occupy the
@@ -79,10 +96,12 @@ inline int32_t bwd_split_target(const distca_ca_params *p) {
 inline SchedGeom dq_geom(const distca_ca_params *p) {
   SchedGeom g = fwd_geom(p);
   g.rows_per_block = kDqRows;
+  g.merge_tiles = merge_short_tasks(p) ? kMergeTilesDq : 0;  // in the list's cost unit, visible keys / kFwdKV
   return g;
 }
 inline SchedGeom bwd_geom(const distca_ca_params *p) {
   SchedGeom g;
+  g.merge_tiles = 0;
   g.rows_per_block = kBwdRows;
   g.kv_per_block = kBwdKV;
   g.group = p->num_heads_q / p->num_heads_kv;

@@ -58,19 +58,22 @@ struct FwdArgs {
   int32_t *tickets;  // one counter per kv head (sched.h)
   const int64_t *q_task_off, *out_task_off;
   int64_t q_tok_bytes, out_tok_bytes;
+  int32_t merge_tiles;   // MERGE kernels: the list's merge_tiles (sched.h)
   int32_t lse_in_token;  // 1: lse of (token, head) as fp32 at token + hq * 256 + h * 4 (the [out | lse] reply), 0: lse[h][token]
   KvShards shards;       // SEG kernels: k and v are the bases of a buffer that holds the stored rows shard by shard
 };
 
 // SEG: K/V rows are addressed through a table of shards (kv_shards.h) instead of as one dense tensor.
-template <int MSUB, bool SEG>
+// MERGE: a work item is several consecutive blocks of a task's query rows (sched.h, fwd_merge), worked off one after the
+// other; otherwise it is one block.
+template <int MSUB, bool SEG, bool MERGE>
 __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 1)) void ca_fwd_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int nitems = a.sched[0];
   int item, kvh;
   if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
   const int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
-  const int task = it.x, mblk = it.y;
+  const int task = it.x;
 
   const int q0 = a.cu_q[task];
   const int lq = a.cu_q[task + 1] - q0;
@@ -79,11 +82,33 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int G = a.group;
   const int shift = lk - lq;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, g = lane >> 5;
   constexpr int kRows = kFwdWaves * 32 * MSUB;
-  const int row_wg = mblk * kRows;
   const int nrows = lq * G;
+  // the blocks of this item
+  int mb_first = it.y, mb_end = it.y + 1;
+  if constexpr (MERGE) {
+    SchedGeom geom;
+    geom.rows_per_block = kRows; geom.kv_per_block = kFwdKV; geom.group = G; geom.causal = a.causal; geom.merge_tiles = a.merge_tiles;
+    const int m = fwd_merge(geom, lq, lk), nblk = (nrows + kRows - 1) / kRows;
+    mb_first = it.y * m;
+    mb_end = mb_first + m < nblk ? mb_first + m : nblk;
+  }
+  // (a jump back rather than a loop statement: without MERGE the body below is then straight-line code, exactly the
+  // kernel that takes one block per item)
+  int mblk = mb_first;
+  // MERGE: the Q rows and the first K tile of a block are requested while the block before it finishes (below)
+  elemx8 qf[MSUB][8];
+  bool requested = false;
+next_block:
+  // MERGE: the thread index is made opaque once per block, so that what derives from it (the lanes' LDS and global
+  // offsets, a few dozen registers) is computed afresh for every block instead of being carried, and partly spilled,
+  // across the whole body: a reload from scratch memory waits for every request in flight, those made for the next
+  // block included.
+  int tid_ = threadIdx.x;
+  if constexpr (MERGE) asm volatile("" : "+v"(tid_));
+  const int tid = tid_, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int row_wg = mblk * kRows;
 
   // ---- KV extent of this workgroup
   int tok_end = (row_wg + kRows + G - 1) / G;
@@ -124,13 +149,14 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   }
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds row l32, d = 16*s + 8*g .. +7
-  elemx8 qf[MSUB][8];
+  if (!MERGE || !requested) {
 #pragma unroll
-  for (int m = 0; m < MSUB; ++m) {
+    for (int m = 0; m < MSUB; ++m) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      if (valid[m]) qf[m][s] = *reinterpret_cast<const elemx8 *>(qptr[m] + 16 * s + 8 * g);
-      else qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+      for (int s = 0; s < 8; ++s) {
+        if (valid[m]) qf[m][s] = *reinterpret_cast<const elemx8 *>(qptr[m] + 16 * s + 8 * g);
+        else qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
     }
   }
 
@@ -369,8 +395,31 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   // waits for its own requests before b(2p+2).  The MFMA halves are the critical path of a period (one
   // group's, then the other's); a request holds its wave for a hundred cycles or so, and in front of
   // group 0's MFMA half that time showed in the period (-3 % with the requests behind it).
+  // MERGE: what the item's next block starts with is requested when this block's tile loop is over, so that it
+  // arrives while the results are normalised and stored: its Q rows (the Q registers are free: every S of this block
+  // is done) and its first K tile (no wave reads a K stage any more: the last barrier of the loop lies behind every S
+  // phase; tile 0 is the same for every block of a task).  The run and cursor objects the request goes through are
+  // set up afresh by the next block, which also finds its tile 0 request made.  (Made from inside the loop's last
+  // period instead, the requests cost the loop its register allocation: six hundred spills.)
+  const bool more = MERGE && mblk + 1 < mb_end;
+  auto request_next_block = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int m = 0; m < MSUB; ++m) {
+      const int nrow = row[m] + kRows;
+      const int ntok = nrow / G;
+      const elem_t *np = reinterpret_cast<const elem_t *>(qbytes + (int64_t)ntok * a.q_tok_bytes) + (kvh * G + (nrow - ntok * G)) * kHeadDim;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        if (nrow < nrows) qf[m][s] = *reinterpret_cast<const elemx8 *>(np + 16 * s + 8 * g);
+        else qf[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    krun = Run{kbase, SEG ? 0 : lk};
+    if constexpr (SEG) kcur.open(a.shards, a.shards.task_shard[task]);
+    issue_k(0);  // (the next block has rows, hence at least one tile)
+  };
   const int grp = uwave >> 2;
-  if (ntiles > 0) issue_k(0);
+  if (ntiles > 0 && (!MERGE || !requested)) issue_k(0);
   wait_vm0();
   __syncthreads();  // b0
   // The period loop is unrolled by two so that the LDS stage of every operand read is a constant folded into
@@ -415,6 +464,19 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     }
   }
 
+  // (Where the results go is worked out ahead of those requests: should the compiler have parked a pointer in scratch
+  // memory, fetching it back afterwards would wait for the requests as well.)
+  uint8_t *otok_m[MSUB];
+#pragma unroll
+  for (int m = 0; m < MSUB; ++m) {
+    otok_m[m] = obytes + (int64_t)tok[m] * a.out_tok_bytes;
+    if constexpr (MERGE) asm volatile("" : "+v"(otok_m[m]));
+  }
+  if constexpr (MERGE) {
+    requested = more;
+    if (more) request_next_block();
+  }
+
   // ---- epilogue: normalise, write O (bf16) and LSE (fp32, natural log)
 #pragma unroll
   for (int m = 0; m < MSUB; ++m) {
@@ -422,7 +484,7 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
-      uint8_t *otok = obytes + (int64_t)tok[m] * a.out_tok_bytes;
+      uint8_t *otok = otok_m[m];
       elem_t *op = reinterpret_cast<elem_t *>(otok) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
@@ -448,6 +510,9 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
         }
       }
     }
+  }
+  if constexpr (MERGE) {
+    if (++mblk < mb_end) goto next_block;
   }
 }
 
@@ -598,6 +663,7 @@ int DISTCA_FN(run_fwd_tokens)(const void *q_base, const int64_t *q_task_off, int
   a.total_q = p->total_q; a.causal = p->causal != 0; a.scale = p->softmax_scale;
   a.q_task_off = q_task_off; a.out_task_off = out_task_off; a.q_tok_bytes = q_tok_bytes; a.out_tok_bytes = out_tok_bytes;
   a.lse_in_token = lse ? 0 : 1;
+  a.merge_tiles = geom.merge_tiles;
   a.shards = KvShards{};
   if (kv_shards) {
     rc = make_kv_shards(kv_shards, kv_off, false, &a.shards);
@@ -606,17 +672,22 @@ int DISTCA_FN(run_fwd_tokens)(const void *q_base, const int64_t *q_task_off, int
   const int64_t grid = max_items * p->num_heads_kv * kSchedOversubNum / kSchedOversubDen;
   if (grid > 0x7fffffff) return fail(DISTCA_E_INVALID, "ca_fwd: grid too large");
   if (device_setup_pending(kSlotFwdLds)) {
-    hipError_t e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ca_fwd_kernel<kFwdMsub, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
-    if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
+    const void *kernels[] = {(const void *)ca_fwd_kernel<kFwdMsub, false, false>, (const void *)ca_fwd_kernel<kFwdMsub, true, false>,
+                             (const void *)ca_fwd_kernel<kFwdMsub, false, true>, (const void *)ca_fwd_kernel<kFwdMsub, true, true>};
+    for (const void *kf : kernels) {
+      hipError_t e = hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds);
+      if (e != hipSuccess) return fail(DISTCA_E_LAUNCH, "ca_fwd: cannot reserve %d B of LDS: %s", kFwdLds, hipGetErrorString(e));
+    }
     device_setup_done(kSlotFwdLds);
   }
   {
     ScopedTimer timer(DISTCA_TIMER_CA_FWD, s);
-    if (kv_shards)
-      hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, true>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
-    else
-      hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, false>), dim3((unsigned)grid), dim3(kFwdWaves * 64), kFwdLds, s, a);
+    const dim3 g((unsigned)grid), b(kFwdWaves * 64);
+    const bool merge = geom.merge_tiles > 0;
+    if (kv_shards && merge) hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, true, true>), g, b, kFwdLds, s, a);
+    else if (kv_shards) hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, true, false>), g, b, kFwdLds, s, a);
+    else if (merge) hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, false, true>), g, b, kFwdLds, s, a);
+    else hipLaunchKernelGGL((ca_fwd_kernel<kFwdMsub, false, false>), g, b, kFwdLds, s, a);
   }
   return check_launch("ca_fwd");
 }

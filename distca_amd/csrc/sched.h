@@ -31,6 +31,8 @@ struct SchedGeom {
                            // many pieces exist per kv head (see piece_count)
   int32_t walk_round;      // backward only, 0 = off: items whose rank in the list is in an odd group of this many
                            // carry kWalkUp (below)
+  int32_t merge_tiles;     // lists over blocks of query rows only, 0 = off: consecutive blocks of a short task form
+                           // one work item, as many as bring it to about this many KV tiles (fwd_merge)
 };
 
 // Walk direction of a dK/dV item.  A key block streams the query rows that see it, and the compute units of one
@@ -94,6 +96,31 @@ DISTCA_HD int32_t fwd_visible_keys(const SchedGeom &g, int32_t lq, int32_t lk, i
 }
 DISTCA_HD int32_t fwd_cost(const SchedGeom &g, int32_t lq, int32_t lk, int32_t i) {
   return ceil_div(fwd_visible_keys(g, lq, lk, i), g.kv_per_block);
+}
+
+// Short tasks: a block of query rows that sees a handful of KV tiles spends a third of its workgroup's time outside the
+// tile loop (drawing its ticket, loading the item and its bounds, waiting for Q and the first tile, draining the
+// output).  With merge_tiles set, every work item of a task is `fwd_merge` consecutive blocks, which one workgroup
+// works off one after the other: the ticket and the task's bounds are paid once, and what the next block needs can
+// be requested while the present one finishes.  The number depends on the task alone (its most expensive block, the
+// last one), so the kernel finds the blocks of item i without a table: blocks i * m .. min((i + 1) * m, blocks) - 1.
+constexpr int32_t kMaxMerge = 8;
+DISTCA_HD int32_t fwd_merge(const SchedGeom &g, int32_t lq, int32_t lk) {
+  if (g.merge_tiles <= 0) return 1;
+  const int32_t n = fwd_num_blocks(g, lq);
+  if (n <= 1) return 1;
+  const int32_t worst = fwd_cost(g, lq, lk, n - 1);
+  int32_t m = g.merge_tiles / (worst > 0 ? worst : 1);
+  return m < 1 ? 1 : (m > kMaxMerge ? kMaxMerge : m);
+}
+DISTCA_HD int32_t fwd_num_items(const SchedGeom &g, int32_t lq, int32_t lk) { return ceil_div(fwd_num_blocks(g, lq), fwd_merge(g, lq, lk)); }
+DISTCA_HD int32_t fwd_item_cost(const SchedGeom &g, int32_t lq, int32_t lk, int32_t i) {
+  const int32_t m = fwd_merge(g, lq, lk);
+  if (m == 1) return fwd_cost(g, lq, lk, i);
+  const int32_t n = fwd_num_blocks(g, lq);
+  int32_t c = 0;
+  for (int32_t b = i * m; b < (i + 1) * m && b < n; ++b) c += fwd_cost(g, lq, lk, b);
+  return c;
 }
 
 // backward: blocks of keys

@@ -37,12 +37,12 @@ struct TaskUnits {
   SchedGeom g;
   __device__ __forceinline__ int32_t blocks(int32_t b) const {
     const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
-    const int32_t n = BWD ? bwd_num_blocks(g, lq, lk) : fwd_num_blocks(g, lq);
+    const int32_t n = BWD ? bwd_num_blocks(g, lq, lk) : fwd_num_items(g, lq, lk);
     return n < 0 ? 0 : n;
   }
   __device__ __forceinline__ int32_t cost(int32_t b, int32_t i) const {
     const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
-    return BWD ? bwd_cost(g, lq, lk, i) : fwd_cost(g, lq, lk, i);
+    return BWD ? bwd_cost(g, lq, lk, i) : fwd_item_cost(g, lq, lk, i);
   }
 };
 struct GroupUnits {
@@ -352,9 +352,9 @@ extern "C" int64_t distca_ca_schedule_host(int kind, const int32_t *cu_q, const 
   unsigned long long total_cost = 0;
   for (int32_t b = 0; b < p->num_tasks; ++b) {
     const int32_t lq = cu_q[b + 1] - cu_q[b], lk = cu_k[b + 1] - cu_k[b];
-    const int32_t n = kind == 0 ? fwd_num_blocks(g, lq) : bwd_num_blocks(g, lq, lk);
+    const int32_t n = kind == 0 ? fwd_num_items(g, lq, lk) : bwd_num_blocks(g, lq, lk);
     for (int32_t i = 0; i < n; ++i) {
-      const int32_t c = kind == 0 ? fwd_cost(g, lq, lk, i) : bwd_cost(g, lq, lk, i);
+      const int32_t c = kind == 0 ? fwd_item_cost(g, lq, lk, i) : bwd_cost(g, lq, lk, i);
       whole.push_back({b, i, c, 0, 0});
       total_cost += (unsigned long long)c;
     }

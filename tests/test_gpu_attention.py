@@ -126,6 +126,17 @@ def test_queries_that_see_no_key(cuda):
     assert torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all() and torch.isfinite(dq.float()).all()
 
 
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4)])
+def test_short_tasks_as_merged_work_items(cuda, hq, hkv):
+    """A batch whose tasks average fewer than 2048 query tokens has the forward and dQ kernels work off several
+    consecutive blocks of a task per work item (eight for the 1024-token document here, whose sixteen blocks at four
+    heads per kv head make two items; the last item of a task is usually shorter), the next block's Q rows and first K
+    tile requested while the present one is normalised and stored.  Whole documents and tasks with prefixes, lengths
+    on and off the block edges."""
+    _run([1024, 1000, 513, 1, 2047, 64], [1024, 1000, 513, 1, 2047, 64], hq, hkv, 51, cuda)
+    _run([1024, 300, 700], [1024, 1324, 764], hq, hkv, 52, cuda)
+
+
 def test_non_causal(cuda):
     _run([100, 260], [100, 260], 4, 2, 6, cuda, causal=False)
 

@@ -30,7 +30,13 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("lq,lk", CASES)
+# Batches of short tasks (fewer than 2048 query tokens per task on average) have the forward and dQ lists made of
+# merged items: item i of a task is its blocks i m .. (i + 1) m - 1, with m = 128 // (KV tiles of the task's last block),
+# between 1 and 8, so that a work item has about 128 tiles to stream whatever the task's length.
+MERGE_MEAN_TOKENS, MERGE_TILES, MAX_MERGE = 2048, 128, 8
+
+
+@pytest.mark.parametrize("lq,lk", CASES + [([4096, 2100], [4096, 5000]), ([1024] * 6, [1024] * 6), ([700, 2500, 90], [900, 2500, 4000])])
 @pytest.mark.parametrize("causal", [True, False])
 def test_forward_items_tile_each_task_once_and_cover_visible_keys(lq, lk, causal):
     rows, kv = scheduler.tile_shape(scheduler.FWD, HQ, HKV)
@@ -39,13 +45,23 @@ def test_forward_items_tile_each_task_once_and_cover_visible_keys(lq, lk, causal
     for t, b, c, w in items.tolist():
         assert (t, b) not in seen and w == 1 << 16          # forward items are never cut
         seen[(t, b)] = c
+    merged = sum(lq) < MERGE_MEAN_TOKENS * len(lq)
+    some_merged = False
     for t, (a, k) in enumerate(zip(lq, lk)):
         nblk = -(-a * G // rows)
-        assert sorted(b for (tt, b) in seen if tt == t) == list(range(nblk))
+        costs = []
         for b in range(nblk):
             last_tok = min(a, -(-(b + 1) * rows // G)) - 1           # last token with a row in the block
             vis = min(k, max(0, last_tok + 1 + (k - a))) if causal else k
-            assert seen[(t, b)] == -(-vis // kv)                       # KV tiles the block streams
+            costs.append(-(-vis // kv))                                # KV tiles the block streams
+        m = min(MAX_MERGE, max(1, MERGE_TILES // max(1, costs[-1]))) if merged and nblk > 1 else 1
+        some_merged |= m > 1
+        nitems = -(-nblk // m)
+        assert sorted(b for (tt, b) in seen if tt == t) == list(range(nitems))
+        for i in range(nitems):
+            assert seen[(t, i)] == sum(costs[i * m:(i + 1) * m])
+    if not merged:
+        assert not some_merged
     costs = items[:, 2]
     assert (np.diff(costs) <= 0).all()
 
@@ -132,9 +148,10 @@ def test_empty_batch_and_empty_tasks():
 def test_group_sizes():
     for hq, hkv in [(8, 8), (16, 8), (64, 8), (28, 4)]:
         rows, kv = scheduler.tile_shape(scheduler.FWD, hq, hkv)
-        items = scheduler.build_schedule(scheduler.FWD, _cu([100, 37]), _cu([100, 37]), hq, hkv)
+        # (tasks long enough that their blocks are not merged into larger work items: one item per block)
+        items = scheduler.build_schedule(scheduler.FWD, _cu([4100, 2037]), _cu([4100, 2037]), hq, hkv)
         g = hq // hkv
-        assert len(items) == -(-100 * g // rows) + -(-37 * g // rows)
+        assert len(items) == -(-4100 * g // rows) + -(-2037 * g // rows)
 
 
 def _check_capacity_and_tiling(lq, lk, hq, hkv, total_k=None):
