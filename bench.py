@@ -35,7 +35,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
 # WRITE_SIZE (x1.000), factors from the pack kernels' known copy sizes in the same run
-MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.92e9, "ca_bwd_dkdv64_kernel": 24.12e9, "ca_bwd_dq64_kernel": 13.46e9}
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.95e9, "ca_bwd_dkdv64_kernel": 22.58e9, "ca_bwd_dq64_kernel": 13.34e9}
 
 
 def log(*a):
@@ -168,7 +168,7 @@ def pack_unpack_bench(torch, dev, iters: int = 10):
     return res
 
 
-def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap: int = 4096):
+def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap: int = 4096, in_place_only: bool = False):
     """The CA server's ticks on the bench workload: every document cut into shards of at most `shard_cap`
     tokens, one CA task per shard reading its document's prefix.  Forward tick = unpack K/V (each stored shard
     once) + attention reading q from the receive buffer and writing [out | lse] tokens into the send buffer;
@@ -231,8 +231,9 @@ def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap:
     fwd_timers, bwd_timers = (_lib.TIMER_CA_FWD,), (_lib.TIMER_CA_BWD_DQ, _lib.TIMER_CA_BWD)
     res["forward_ms"], res["forward_attention_kernel_ms"] = timed_with_kernels(
         lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det), fwd_timers)
-    res["forward_kv_unpacked_ms"], res["forward_kv_unpacked_attention_kernel_ms"] = timed_with_kernels(
-        lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det, kv_shards_in_place=False), fwd_timers)
+    if not in_place_only:
+        res["forward_kv_unpacked_ms"], res["forward_kv_unpacked_attention_kernel_ms"] = timed_with_kernels(
+            lambda: ca_server_forward(recv, send, fmeta, fa_params, fa_det, kv_shards_in_place=False), fwd_timers)
     out, lse = ca_server_forward(recv, send, fmeta, fa_params, fa_det, in_place=False)
     del recv, send
     request = TokenLayout.of([flat(do), out, lse.T.contiguous(), flat(q)]).merge([flat(do), out, lse.T.contiguous(), flat(q)])
@@ -244,8 +245,10 @@ def server_tick_bench(torch, dev, batch, q, k, v, do, iters: int = 4, shard_cap:
     bwd = lambda **kw: ca_server_backward(recv, send, bmeta, fa_det, fa_params.cu_seqlens_q, fa_params.cu_seqlens_kv,
                                           fa_params.max_seqlen_q, fa_params.max_seqlen_kv, **kw)
     res["backward_ms"], res["backward_attention_kernels_ms"] = timed_with_kernels(lambda: bwd(), bwd_timers)
-    res["backward_kv_unpacked_ms"], res["backward_kv_unpacked_attention_kernels_ms"] = timed_with_kernels(
-        lambda: bwd(kv_shards_in_place=False), bwd_timers)
+    if not in_place_only:
+        res["backward_kv_unpacked_ms"], res["backward_kv_unpacked_attention_kernels_ms"] = timed_with_kernels(
+            lambda: bwd(kv_shards_in_place=False), bwd_timers)
+    res["ticks_timed_per_form"] = iters + 2
     res["note"] = ("deterministic ticks (the reference's default).  forward_ms / backward_ms: everything in place: query and "
                    "request tokens and K/V shards read where they lie in the receive buffer, [out | lse], dq and the shards' "
                    "dk / dv written where they belong in the send buffer, no pack kernel; *_kv_unpacked_ms: every stored K/V "
@@ -263,7 +266,8 @@ def mfma_probe(torch, _lib, dev, executed_tflops: float, rounds: int = 5, warm_s
     scratch = torch.zeros(4, dtype=torch.int64, device=dev)
     stream_ptr = torch.cuda.current_stream().cuda_stream
     kinds = (("mfma_only", _lib.PROBE_MFMA_ONLY), ("with_1kb_lds_read_per_mfma", _lib.PROBE_LDS_READ),
-             ("with_4_fma_per_mfma", _lib.PROBE_FMA4), ("with_2_exp_per_mfma", _lib.PROBE_EXP2))
+             ("with_4_fma_per_mfma", _lib.PROBE_FMA4), ("with_2_exp_per_mfma", _lib.PROBE_EXP2),
+             ("with_attention_side_work", _lib.PROBE_MIX))
     iters = 20000
     for _, kind in kinds:    # the first launch of a kernel also loads it
         _lib.probe_mfma_rate(kind, 200, scratch.data_ptr(), stream_ptr)
@@ -282,6 +286,9 @@ def mfma_probe(torch, _lib, dev, executed_tflops: float, rounds: int = 5, warm_s
                        "clock_GHz": round(float(np.median([r[2] for r in runs[name]])), 3)}
     probe["executed_TFLOP/s_of_the_three_attention_kernels"] = round(executed_tflops, 1)
     probe["executed_over_mfma_only"] = round(executed_tflops / probe["mfma_only"]["TFLOP/s"], 4)
+    # with_attention_side_work: beside every MFMA half of a 1 KB LDS read, two multiply-adds, half an exponential and half
+    # a conversion, the per-MFMA average of the backward kernels' tile loops (no tile requests, barriers or prologues)
+    probe["executed_over_mfma_with_attention_side_work"] = round(executed_tflops / probe["with_attention_side_work"]["TFLOP/s"], 4)
     probe["note"] = (f"v_mfma_f32_32x32x16_bf16 on pseudo-random operands, one wave per SIMD on every SIMD, {8 * iters} per wave and run; "
                      f"{warm_seconds} s of the MFMA-only loop first, then the four variants interleaved for {rounds} rounds: median (min..max) "
                      "rate by HIP events, clock by the device's cycle and real-time counters: what the power limit leaves "
@@ -353,6 +360,8 @@ def main():
     ap.add_argument("--no-tick", action="store_true")
     ap.add_argument("--no-probe", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other attention configurations (cfg3b, cfg5, short tasks)")
+    ap.add_argument("--tick-in-place-only", action="store_true",
+                    help="server-tick leg: only the all-in-place ticks (for a kernel trace that shows them without pack kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the CA-server path; --gpus must be 1 "
@@ -424,7 +433,10 @@ def main():
         probe = mfma_probe(torch, _lib, dev, executed)
         log(f"  MFMA-only loop {probe['mfma_only']['TFLOP/s']} TFLOP/s (median of {probe['rounds']} rounds, {probe['mfma_only']['TFLOP/s_min']}"
             f"..{probe['mfma_only']['TFLOP/s_max']}) at {probe['mfma_only']['clock_GHz']} GHz; the attention kernels execute "
-            f"{probe['executed_TFLOP/s_of_the_three_attention_kernels']} TFLOP/s = {100 * probe['executed_over_mfma_only']:.1f} % of it")
+            f"{probe['executed_TFLOP/s_of_the_three_attention_kernels']} TFLOP/s = {100 * probe['executed_over_mfma_only']:.1f} % of it, "
+            f"{100 * probe['executed_over_mfma_with_attention_side_work']:.1f} % of the loop with the backward's per-MFMA side work "
+            f"({probe['with_attention_side_work']['TFLOP/s']} TFLOP/s at {probe['with_attention_side_work']['clock_GHz']} GHz, "
+            f"{probe['with_attention_side_work']['cycles_per_mfma']} cycles per MFMA)")
 
     pack = None
     if not args.no_pack:
@@ -438,11 +450,11 @@ def main():
 
     tick = None
     if not args.no_tick:
-        tick = server_tick_bench(torch, dev, batch, q, k, v, do)
+        tick = server_tick_bench(torch, dev, batch, q, k, v, do, in_place_only=args.tick_in_place_only)
         log(f"  server tick over {tick['tasks']} tasks: forward {tick['forward_ms']} ms (kernel {tick['forward_attention_kernel_ms']}; "
-            f"K/V unpacked first: {tick['forward_kv_unpacked_ms']}, kernel {tick['forward_kv_unpacked_attention_kernel_ms']}), "
+            f"K/V unpacked first: {tick.get('forward_kv_unpacked_ms')}, kernel {tick.get('forward_kv_unpacked_attention_kernel_ms')}), "
             f"backward {tick['backward_ms']} ms (kernels {tick['backward_attention_kernels_ms']}; K/V unpacked first: "
-            f"{tick['backward_kv_unpacked_ms']}, kernels {tick['backward_kv_unpacked_attention_kernels_ms']})")
+            f"{tick.get('backward_kv_unpacked_ms')}, kernels {tick.get('backward_kv_unpacked_attention_kernels_ms')})")
 
     extra = None
     if not args.no_extra:

@@ -115,12 +115,13 @@ def timing_read(which: int):
     return ms.value, n.value
 
 
-PROBE_MFMA_ONLY, PROBE_LDS_READ, PROBE_FMA4, PROBE_EXP2 = range(4)
+PROBE_MFMA_ONLY, PROBE_LDS_READ, PROBE_FMA4, PROBE_EXP2, PROBE_MIX = range(5)
 
 
 def probe_mfma_rate(kind: int, iters: int, scratch_ptr: int, stream_ptr: int = 0):
     """(TFLOP/s, cycles per MFMA, shader clock in GHz) of a loop of MFMAs on every SIMD of the device, with
-    nothing (PROBE_MFMA_ONLY), an LDS read, four FMAs or two exponentials behind every MFMA.  `scratch_ptr`: 32
+    nothing (PROBE_MFMA_ONLY), an LDS read, four FMAs, two exponentials, or the attention backward's average side
+    work (PROBE_MIX) behind every MFMA.  `scratch_ptr`: 32
     bytes of device memory.  Synchronises the stream."""
     tf, cyc, ghz = ctypes.c_double(0), ctypes.c_double(0), ctypes.c_double(0)
     check(load().distca_probe_mfma_rate(kind, iters, scratch_ptr, ctypes.byref(tf), ctypes.byref(cyc), ctypes.byref(ghz),

@@ -15,7 +15,9 @@ namespace {
 
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
 
-enum { kProbeMfmaOnly = 0, kProbeLdsRead = 1, kProbeFma4 = 2, kProbeExp2 = 3, kProbeKinds = 4 };
+// kProbeMix: beside every MFMA what the backward kernels have beside theirs, on average: half a kilobyte of LDS operand
+// reads (one 1 KB read per two MFMAs), two multiply-adds, half an exponential and half a conversion to bf16 pairs.
+enum { kProbeMfmaOnly = 0, kProbeLdsRead = 1, kProbeFma4 = 2, kProbeExp2 = 3, kProbeMix = 4, kProbeKinds = 5 };
 
 template <int KIND>
 __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(int iters, unsigned long long *out) {
@@ -44,6 +46,7 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(int iters, unsigned l
 #pragma unroll
   for (int i = 0; i < 8; ++i) x[i] = 0.001f * (lane + i);
   f32x4 ld[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+  uint32_t pk = 0;
   const uint32_t addr = (uint32_t)(uintptr_t)(DISTCA_LDS uint32_t *)tile + lane * 16;
   const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
   for (int it = 0; it < iters; ++it) {
@@ -59,6 +62,13 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(int iters, unsigned l
 #pragma unroll
         for (int j = 0; j < 2; ++j) asm volatile("v_exp_f32 %0, %0" : "+v"(x[(m * 2 + j) & 7]));
       }
+      if (KIND == kProbeMix) {
+        if (m & 1) asm volatile("ds_read_b128 %0, %1" : "=v"(ld[(m >> 1) & 1]) : "v"(addr));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(x[(m * 2 + j) & 7]) : "v"(y));
+        if (m & 1) asm volatile("v_exp_f32 %0, %0" : "+v"(x[m & 7]));
+        else asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pk) : "v"(x[m & 7]), "v"(x[(m + 1) & 7]));
+      }
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -70,7 +80,7 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(int iters, unsigned l
     for (int r = 0; r < 16; ++r) t += acc[m][r];
 #pragma unroll
   for (int i = 0; i < 8; ++i) t += x[i];
-  t += ld[0][0] + ld[1][3];
+  t += ld[0][0] + ld[1][3] + (float)pk;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     out[0] = c1 - c0;
     out[1] = r1 - r0;
@@ -98,7 +108,8 @@ extern "C" int distca_probe_mfma_rate(int kind, int iters, void *scratch32, doub
     case kProbeMfmaOnly: hipLaunchKernelGGL((mfma_rate_kernel<kProbeMfmaOnly>), dim3(cus), dim3(256), 0, s, iters, out); break;
     case kProbeLdsRead: hipLaunchKernelGGL((mfma_rate_kernel<kProbeLdsRead>), dim3(cus), dim3(256), 0, s, iters, out); break;
     case kProbeFma4: hipLaunchKernelGGL((mfma_rate_kernel<kProbeFma4>), dim3(cus), dim3(256), 0, s, iters, out); break;
-    default: hipLaunchKernelGGL((mfma_rate_kernel<kProbeExp2>), dim3(cus), dim3(256), 0, s, iters, out); break;
+    case kProbeExp2: hipLaunchKernelGGL((mfma_rate_kernel<kProbeExp2>), dim3(cus), dim3(256), 0, s, iters, out); break;
+    default: hipLaunchKernelGGL((mfma_rate_kernel<kProbeMix>), dim3(cus), dim3(256), 0, s, iters, out); break;
   }
   (void)hipEventRecord(e1, s);
   int rc = check_launch("probe_mfma_rate");

@@ -361,7 +361,9 @@ int distca_timing_read(int which, double *total_ms, int64_t *launches);
  * diagnostic for benchmarks, which print it beside the kernels' own rate.  One
  * wave on every SIMD issues 8 * iters v_mfma_f32_32x32x16_bf16 on pseudo-random
  * operands and, behind every MFMA, nothing (kind 0), one 1 KB LDS read (1),
- * four v_fma_f32 (2) or two v_exp_f32 (3): work that fits into the MFMA's
+ * four v_fma_f32 (2), two v_exp_f32 (3), or (4) what the attention backward has
+ * beside an MFMA on average: half of a 1 KB LDS read, two v_fma_f32, half a
+ * v_exp_f32 and half a v_cvt_pk_bf16_f32.  All of it fits into the MFMA's
  * shadow, so that the pipe stays fully occupied and the result shows what the
  * power limit leaves of the clock.  Returns the MFMA rate in TFLOP/s (by HIP
  * events on `stream`), the cycles per MFMA and the shader clock in GHz (by the

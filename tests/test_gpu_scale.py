@@ -579,7 +579,7 @@ def test_mfma_rate_probe(cuda):
     printed."""
     from distca_amd import _lib
     scratch = torch.zeros(4, dtype=torch.int64, device=cuda)
-    for kind in (_lib.PROBE_MFMA_ONLY, _lib.PROBE_LDS_READ, _lib.PROBE_FMA4, _lib.PROBE_EXP2):
+    for kind in (_lib.PROBE_MFMA_ONLY, _lib.PROBE_LDS_READ, _lib.PROBE_FMA4, _lib.PROBE_EXP2, _lib.PROBE_MIX):
         _lib.probe_mfma_rate(kind, 2000, scratch.data_ptr())   # the first launch of a kernel also loads it
         tf, cyc, ghz = _lib.probe_mfma_rate(kind, 40000, scratch.data_ptr())
         print(f"probe kind {kind}: {tf:.0f} TFLOP/s, {cyc:.1f} cycles per MFMA, {ghz:.2f} GHz", flush=True)
