@@ -16,6 +16,8 @@ reference derives the same quantities for any number of ranks from planner outpu
 """
 from __future__ import annotations
 
+import warnings
+
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple, Union
 
@@ -162,6 +164,15 @@ class SharedKVLayout:
     entry_of_stored: Tensor   # int64 [stored shards]: the K/V entry (first of its aliases) it is unpacked from
     kv_task_offsets: Tensor   # int32 [tasks]: first store row of each task's prefix
     num_rows: int
+
+
+def _warn_no_shared_layout():
+    """Said once per call site that drops the one-copy layout: the ticks then still give the same results, through the
+    reference's layout (a copy of the prefix per task, the duplicate-gradient sum, a masked pack), at the cost of the
+    duplicated K/V rows."""
+    warnings.warn("the K/V shards of this step's tasks are not nested prefixes of one stored sequence per document: "
+                  "the server ticks keep one K/V copy per task (unpack, duplicate-gradient sum, masked pack) instead of "
+                  "reading one stored copy in place", RuntimeWarning, stacklevel=3)
 
 
 def shared_kv_layout(task_kv_lens: Sequence[int], entry_tokens: Sequence[int], entry_key: Sequence[int]) -> Optional[SharedKVLayout]:
@@ -358,6 +369,8 @@ def server_metas(plan: SingleRankPlan, device="cuda", shared_kv: bool = True):
     fwd = ServerFwdMeta(i64(plan.q_seqlens), i64(plan.kv_entry_tokens), i64(fq), i64(fk), i64(fv),
                         i64(plan.q_seqlens), i64(fo), (tq, hq_d), (tk, hkv_d))
     shared = shared_kv_layout(plan.kv_seqlens.tolist(), plan.kv_entry_tokens.tolist(), plan.kv_entry_shard.tolist()) if shared_kv else None
+    if shared_kv and shared is None:
+        _warn_no_shared_layout()
     if shared is not None:
         fwd.shared_kv = SharedKVOnDevice.build(shared, fk, fv, device)
     bq, bk, bv, b_recv = plan.request_layout(True)
@@ -413,6 +426,7 @@ class PingPangSingleStepPackedSeqParams:
             lens = host(cu).diff().tolist()
             layout = shared_kv_layout(lens, host(req.seq_lens[1].recv_seqlens).tolist(), k_off.tolist())
             if layout is None:
+                _warn_no_shared_layout()
                 out.append(None)
                 continue
             gk = gv = None

@@ -2,7 +2,10 @@
 document cut into shards a | b | c (compute_metadata.py:404-459,202-273,277-323 of the
 reference, world size 1): tasks Lq = [a, b, c], Lk = [a, a+b, a+b+c]; K/V entries
 [k0 | k0 k1 | k0 k1 k2]; main copies are the first occurrences; duplicates are summed into them."""
+import warnings
+
 import numpy as np
+import pytest
 import torch
 
 from distca_amd import metadata
@@ -143,3 +146,21 @@ def test_shared_kv_layout_keeps_one_copy_per_shard_and_documents_contiguous():
     assert shared_kv_layout([8, 5], [3, 5, 3, 2], [0, 1, 0, 2]) is None
     # entries that do not add up to the task lengths
     assert shared_kv_layout([4], [3], [0]) is None
+
+
+def test_a_step_without_nested_prefixes_says_that_it_keeps_a_copy_per_task(monkeypatch):
+    """When the K/V shards of a step's tasks are not nested prefixes of one stored sequence per document, the one-copy
+    layout does not exist: the step carries none (the ticks then take the reference's layout) and says so once."""
+    p = metadata.single_rank_plan([[3, 5], [4]], 4, 2)
+    step = metadata.single_rank_step_params(p)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        dev = step.to_device("cpu")          # nested prefixes: no warning, both layouts present
+    assert dev.shared_kv_fwd is not None and dev.shared_kv_bwd is not None
+    monkeypatch.setattr(metadata, "shared_kv_layout", lambda *a, **k: None)
+    with pytest.warns(RuntimeWarning, match="one K/V copy per task"):
+        dev = step.to_device("cpu")
+    assert dev.shared_kv_fwd is None and dev.shared_kv_bwd is None
+    with pytest.warns(RuntimeWarning, match="one K/V copy per task"):
+        _, fwd, bwd, _ = metadata.server_metas(p, device="cpu")
+    assert fwd.shared_kv is None and bwd.shared_kv is None
