@@ -609,8 +609,8 @@ def test_fused_comm_attn_autograd_function(cuda):
 
 @pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4)])
 def test_kv_shards_read_in_place_equal_dense_tensors(cuda, hq, hkv):
-    """distca_ca_fwd_buffers / distca_ca_bwd_buffers with K/V shards of odd lengths (1 to 300 rows: tiles of 32 and 64
-    keys and key blocks of 256 straddle them every which way) scattered through a buffer in shuffled order, K and V in
+    """distca_ca_fwd_buffers / distca_ca_bwd_buffers with K/V shards of odd lengths (0 to 300 rows: tiles of 32 and 64
+    keys and key blocks of 256 straddle them every which way, empty shards in between) scattered through a buffer in shuffled order, K and V in
     separate places, with unused bytes between them: out, lse, dq, and dk / dv gathered back from the shards' places in
     the gradient buffer, are bit for bit what the entry points over dense tensors with kv_task_offsets give
     (deterministic backward; the arithmetic is the same, only the addresses differ), rows that no task reads come back
@@ -629,12 +629,14 @@ def test_kv_shards_read_in_place_equal_dense_tensors(cuda, hq, hkv):
     q_lens = np.array([255, 2, 443, 33, 212, 64, 100], dtype=np.int64)
     kv_off = np.array([doc_start[t] for t in task_doc], dtype=np.int32)
     # shards: every document cut at random places
-    shard_len = []
+    shard_len = [0]                                     # empty shards (padding entries of a plan) lie anywhere in the table
     for n in doc_rows:
         left = n
         while left > 0:
             c = int(min(left, rng.integers(1, 301)))
             shard_len.append(c); left -= c
+            if rng.integers(0, 3) == 0:
+                shard_len.append(0)
     shard_len = np.array(shard_len, dtype=np.int64)
     ns = len(shard_len)
     row_start = np.concatenate([[0], np.cumsum(shard_len)]).astype(np.int32)
