@@ -69,9 +69,11 @@ __device__ __forceinline__ void fence() { __builtin_amdgcn_sched_barrier(0); }
 // and which fill that file exactly.  The S and dP accumulators, which the vector ALU reads and overwrites, must
 // live in the ordinary vector registers instead, and the only way to say so per instruction is to write those
 // MFMAs as assembly with vector-register operands.  The compiler does not know what such a statement executes and
-// so does not space its result from the vector instructions that read it (11 quad-cycles for this MFMA): the
-// order of a block's instructions below keeps at least one later MFMA, which cannot start before the pipe has
-// finished with the one in question, between every such MFMA and the first read of its result.
+// so does not space its result from the vector instructions that read it (an eight-pass MFMA: 11 quad-cycles from
+// its issue): the order of a block's instructions below, held in place by the scheduling fences, keeps between every
+// such MFMA and the first read of its result either two later MFMAs, or one later MFMA (which cannot start before
+// the pipe has finished the eight passes of the one in question) and at least four vector instructions.  Nowhere is
+// a single MFMA the only separation; a change to the block body has to keep that.
 __device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }

@@ -47,7 +47,10 @@ __device__ __forceinline__ void fence() { __builtin_amdgcn_sched_barrier(0); }
 // The S and dP accumulators are read and overwritten by the vector ALU and must live in vector registers; this file
 // is compiled with the compiler's default MFMA form (results in the accumulation registers, right for dQ), so
 // these MFMAs are written as assembly.  The compiler does not space such an instruction from the vector
-// instructions that read its result: the order below keeps a later MFMA, or enough other instructions, between.
+// instructions that read its result (an eight-pass MFMA: 11 quad-cycles from its issue): the order of a tile's
+// instructions below, held in place by the scheduling fences, keeps between every such MFMA and the first read of its
+// result either two later MFMAs, or one later MFMA (which cannot start before the pipe has finished the eight passes
+// of the one in question) and at least four vector instructions; a change to the tile body has to keep that.
 __device__ __forceinline__ void mfma32_v(f32x16 &acc, elemx8 a, elemx8 b) {
   asm volatile(DISTCA_MFMA32_ASM " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
