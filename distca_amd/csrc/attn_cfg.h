@@ -48,7 +48,10 @@ inline int validate_params(const distca_ca_params *p) {
 // Batches of short tasks have the forward and dQ kernels work off several consecutive blocks of a task per work item
 // (sched.h, fwd_merge).  Whether a batch is one is decided from host-known sizes, the mean task length: the kernels
 // built for merged items carry a loop around their body, which the ones for long tasks are spared.
-constexpr int32_t kMergeMeanTokens = 2048;  // batches whose tasks average fewer query tokens than this
+#ifndef DISTCA_MERGE_MEAN_TOKENS
+#define DISTCA_MERGE_MEAN_TOKENS 2048
+#endif
+constexpr int32_t kMergeMeanTokens = DISTCA_MERGE_MEAN_TOKENS;  // batches whose tasks average fewer query tokens than this
 #ifndef DISTCA_MERGE_TILES_FWD
 #define DISTCA_MERGE_TILES_FWD 128
 #endif
