@@ -84,12 +84,20 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
   const int task = it4.x;
 
-  const int q0 = a.cu_q[task];
-  const int64_t qs_task = a.qs_task_off ? a.qs_task_off[task] : (int64_t)q0 * a.qs_tok_bytes;
-  const int64_t dq_task = a.dq_task_off ? a.dq_task_off[task] : (int64_t)q0 * a.dq_tok_bytes;
-  const int lq = a.cu_q[task + 1] - q0;
-  const int lk = a.cu_k[task + 1] - a.cu_k[task];
-  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
+  // The task's bounds and offsets: every load is issued before the first is used (the optional arrays are read
+  // through a pointer that falls back to a place that is always readable, instead of under a branch each: with a
+  // branch per array the loads went to memory one after the other, six trips before the kernel could start).
+  const int32_t *cq = a.cu_q + task, *ck = a.cu_k + task;
+  const int32_t *kvp = a.kv_off ? a.kv_off + task : ck;
+  const int64_t *spare = reinterpret_cast<const int64_t *>(a.zero_row);
+  const int64_t *qsp = a.qs_task_off ? a.qs_task_off + task : spare, *dqp = a.dq_task_off ? a.dq_task_off + task : spare;
+  const int q0 = cq[0], q1 = cq[1], k0 = ck[0], k1 = ck[1], ks = *kvp;
+  const int64_t qs_given = *qsp, dq_given = *dqp;
+  fence();
+  const int64_t qs_task = a.qs_task_off ? qs_given : (int64_t)q0 * a.qs_tok_bytes;
+  const int64_t dq_task = a.dq_task_off ? dq_given : (int64_t)q0 * a.dq_tok_bytes;
+  const int lq = q1 - q0;
+  const int lk = k1 - k0;
   const int G = a.group;
   const int shift = lk - lq;
 
@@ -128,42 +136,46 @@ next_block:
   float lse2[2], delta[2];
   accop_t qf[2][8];
   elemx8 dof[2][8];
+  // All 50 loads of the lane's two rows (Q, dO, O: eight each, and lse) are issued before the first of them is used.
+  // The statements that move Q into the accumulation registers are opaque to the compiler, which orders memory
+  // accesses around every one of them: written load by load, each load waited for the one before it, 32 trips to
+  // memory per block (15 us of the 38 a block of a 1024-token document took).
+  elemx8 qt[2][8], ot[2][8];
+  float lse_row[2];
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
     row[m] = row_wg + (wave * 2 + m) * 32 + l32;
     valid[m] = row[m] < nrows;
-    tok[m] = row[m] / G;
-    const int hg = row[m] - tok[m] * G;
+    // A row past the task (the last block of a task only) reads the task's last row instead, without a branch: with
+    // lse2 = +inf its P and dS are zero whatever Q and dO hold, as long as they are finite, and nothing of it is stored.
+    const int rc = valid[m] ? row[m] : nrows - 1;
+    tok[m] = rc / G;
+    const int hg = rc - tok[m] * G;
     int lm = a.causal ? tok[m] + shift : lk - 1;
     if (lm > lk - 1) lm = lk - 1;
     lim[m] = lm;
     const int64_t ro = qs_task + (int64_t)tok[m] * a.qs_tok_bytes + ((kvh * G + hg) * kHeadDim + 8 * g) * 2;  // bytes
-    lse2[m] = INFINITY;  // rows past the task: P = exp2(-inf) = 0
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      qt[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s);
+      dof[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
+      ot[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.out) + ro + 32 * s);
+    }
+    lse_row[m] = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
+                           : a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]];
+  }
+  fence();
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
     float part = 0.f;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      if (valid[m]) {
-        qf[m][s] = to_acc_regs(*reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.q) + ro + 32 * s));
-        dof[m][s] = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.dout) + ro + 32 * s);
-        const elemx8 of = *reinterpret_cast<const elemx8 *>(reinterpret_cast<const uint8_t *>(a.out) + ro + 32 * s);
+      qf[m][s] = to_acc_regs(qt[m][s]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)of[i];
-      } else {
-        qf[m][s] = to_acc_regs(elemx8{0, 0, 0, 0, 0, 0, 0, 0});
-        dof[m][s] = elemx8{0, 0, 0, 0, 0, 0, 0, 0};
-      }
+      for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)ot[m][s][i];
     }
     delta[m] = pair_sum(part);  // this lane's half of d, then the sum of the lane pair
-    if (valid[m]) {
-      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
-      const float l = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
-                                : a.lse[so];
-      lse2[m] = l * kLog2e;
-      if (g == 0) {
-        a.lse2_w[so] = lse2[m];
-        a.dscaled_w[so] = -delta[m];  // the start value of the dP accumulators in the dK/dV kernel
-      }
-    }
+    lse2[m] = valid[m] ? lse_row[m] * kLog2e : INFINITY;  // rows past the task: P = exp2(-inf) = 0
   }
   // -delta of the lane's row in all 16 registers of a vector: the C operand of a tile's first dP MFMA, so that
   // dS = P * (what the MFMAs leave) costs one instruction per element
@@ -446,11 +458,18 @@ next_block:
   for (; p < ntiles; ++p) advance(p);
   wait_vm<0>();  // nothing may still be on its way into LDS when the workgroup ends
 
-  // ---- epilogue: dQ rows (registers 4*cq..+3 of block db hold d0..d0+3)
+  // ---- epilogue: the row statistics for the dK/dV kernel, which runs after this one (stored here rather than where
+  // they are made: the wait that precedes the tile loop would have to see the stores through as well), and the dQ rows
+  // (registers 4*cq..+3 of block db hold d0..d0+3)
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
     if (valid[m]) {
       const int hg = row[m] - tok[m] * G;
+      if (g == 0) {
+        const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
+        a.lse2_w[so] = lse2[m];
+        a.dscaled_w[so] = ndl[m][0];  // -delta: the start value of the dP accumulators in the dK/dV kernel
+      }
       elem_t *op = reinterpret_cast<elem_t *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
