@@ -503,26 +503,43 @@ next_block:
   wait_vm<0>();  // nothing may still be on its way into LDS when the workgroup ends
 
   // ---- epilogue: the row statistics for the dK/dV kernel, which runs after this one (stored here rather than where
-  // they are made: the wait that precedes the tile loop would have to see the stores through as well), and the dQ rows
-  // (registers 4*cq..+3 of block db hold d0..d0+3)
+  // they are made: the wait that precedes the tile loop would have to see the stores through as well), and the dQ rows.
+  // A lane holds half of each of its two rows in pieces of 8 bytes (registers 4*cq..+3 of block db hold d0..d0+3):
+  // stored from there, an instruction touched 32 rows.  The pieces go to the wave's 16 KB behind the ring instead, in
+  // the tiles' swizzled row layout, and leave from there four whole rows per instruction.
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
-    if (valid[m]) {
+    if (valid[m] && g == 0) {
       const int hg = row[m] - tok[m] * G;
-      if (g == 0) {
-        const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
-        a.lse2_w[so] = lse2[m];
-        a.dscaled_w[so] = ndl[m][0];  // -delta: the start value of the dP accumulators in the dK/dV kernel
-      }
-      elem_t *op = reinterpret_cast<elem_t *>(reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)tok[m] * a.dq_tok_bytes) + (kvh * G + hg) * kHeadDim;
+      const int64_t so = (int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m];
+      a.lse2_w[so] = lse2[m];
+      a.dscaled_w[so] = ndl[m][0];  // -delta: the start value of the dP accumulators in the dK/dV kernel
+    }
+  }
+  {
+    const uint32_t out_b = lds0 + kLdsRing + wave * kStageBytes;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
-          const int d0 = 16 * db + 64 * (cq >> 1) + 8 * (cq & 1) + 4 * g;
-          *reinterpret_cast<elemx4 *>(op + d0) = cvt4(dqacc[m][db][4 * cq] * a.scale, dqacc[m][db][4 * cq + 1] * a.scale,
-                                                      dqacc[m][db][4 * cq + 2] * a.scale, dqacc[m][db][4 * cq + 3] * a.scale);
+          const int chunk = 2 * db + 8 * (cq >> 1) + (cq & 1);  // d0 / 8 with d0 = 16 db + 64 (cq >> 1) + 8 (cq & 1) + 4 g
+          *static_cast<DISTCA_LDS elemx4 *>(const_cast<DISTCA_LDS void *>(lds_ptr(out_b + (32 * m + l32) * kRow + ((chunk ^ tile_swz(l32)) << 4) + 8 * g))) =
+              cvt4(dqacc[m][db][4 * cq] * a.scale, dqacc[m][db][4 * cq + 1] * a.scale, dqacc[m][db][4 * cq + 2] * a.scale,
+                   dqacc[m][db][4 * cq + 3] * a.scale);
         }
+    // (LDS operations of one wave complete in order: the reads below see the writes above)
+    uint8_t *dq_blk = reinterpret_cast<uint8_t *>(a.dq) + dq_task + (int64_t)kvh * G * kHeadDim * 2;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = 4 * i + (lane >> 4);
+      const int rg = wrow0 + r;
+      const elemx8 v = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(out_b + r * kRow + ((lane & 15) << 4)));
+      if (rg < nrows) {
+        const int t = div_group(rg);
+        *reinterpret_cast<elemx8 *>(dq_blk + (int64_t)t * a.dq_tok_bytes + (rg - t * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(r)) << 4)) = v;
+      }
     }
   }
   if constexpr (MERGE) {
