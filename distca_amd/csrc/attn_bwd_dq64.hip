@@ -33,7 +33,9 @@ constexpr int kTile = kKeys * kRow;
 constexpr int kStageBytes = 2 * kTile;  // K tile, V tile
 constexpr int kStages = 4;
 constexpr int kLdsRing = kStages * kStageBytes;
-constexpr int kLds = 2 * kLdsRing;         // the ring, and as much again where a block's dO rows pass through on their way in
+constexpr int kRowsLds = 3 * kTile;        // per wave, behind the ring: 32 rows of Q, dO and O on their way in, 64 rows of dQ on their way out
+constexpr int kLds = kLdsRing + 4 * kRowsLds;
+static_assert(kLds <= 160 * 1024 && kRowsLds >= 64 * kRow, "LDS of a compute unit");
 constexpr int kLoadsPerTile = 4;        // vector-memory instructions a wave issues per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kLead = 2;                // fragments by which sub-block 0 leads in the dQ step
@@ -134,112 +136,6 @@ next_block:
   const uint32_t lds0 = (uint32_t)(uintptr_t)(DISTCA_LDS uint8_t *)lds;
   auto div_group = [&](int n) { return a.group_magic ? (int)__umulhi((uint32_t)n, a.group_magic) : n; };
 
-  // ---- this lane's two rows: Q and dO as B operands (row l32 of a sub-block, d = 16 s + 8 g .. +7), statistics
-  int row[2], tok[2], lim[2];
-  bool valid[2];
-  float lse2[2], delta[2];
-  accop_t qf[2][8];
-  elemx8 dof[2][8];
-  // The wave's 64 rows of Q, dO and O (16 KB each) come through LDS: LDS-direct loads bring four whole rows of 256
-  // bytes per instruction, and the lanes then read their operand fragments (row l32 of a sub-block, chunk 2 s + g) from
-  // there.  Loaded straight into the operand layout, every load instruction touched 32 rows, 32 bytes of each, and the
-  // address unit takes about a cycle per cache line it has to look up: 48 such loads per wave took 7.7 us to *issue*,
-  // a third of what a block of a 1024-token document then spent in its tile loop.  Q goes to the wave's own stage of
-  // the tile ring and dO to the 16 KB behind the ring that belong to the wave, one after the other without a wait in
-  // between; O follows into the first place once Q has been read.  Each wave reads only what it has loaded itself.
-  // Before that, and also in one batch, the lse of the lane's two rows (the opaque statements that move Q into the
-  // accumulation registers order memory accesses around themselves: no load may be left between them).
-  float lse_row[2];
-#pragma unroll
-  for (int m = 0; m < 2; ++m) {
-    row[m] = row_wg + (wave * 2 + m) * 32 + l32;
-    valid[m] = row[m] < nrows;
-    // A row past the task (the last block of a task only) reads the task's last row instead, without a branch: with
-    // lse2 = +inf its P and dS are zero whatever Q and dO hold, as long as they are finite, and nothing of it is stored.
-    const int rc = valid[m] ? row[m] : nrows - 1;
-    tok[m] = div_group(rc);
-    const int hg = rc - tok[m] * G;
-    int lm = a.causal ? tok[m] + shift : lk - 1;
-    if (lm > lk - 1) lm = lk - 1;
-    lim[m] = lm;
-    lse_row[m] = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
-                           : a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]];
-  }
-  const int wrow0 = row_wg + wave * 64;
-  {
-    // offsets from the block's first token: instruction i brings rows 4 i + lane / 16 of the wave, lane % 16 the
-    // position of the 16-byte chunk in the (swizzled) LDS row
-    const int tok0 = div_group(row_wg);
-    const int64_t blk = qs_task + (int64_t)tok0 * a.qs_tok_bytes + (int64_t)kvh * G * kHeadDim * 2;
-    const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + blk, *dob = reinterpret_cast<const uint8_t *>(a.dout) + blk,
-                  *ob = reinterpret_cast<const uint8_t *>(a.out) + blk;
-    uint32_t roff[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int r = 4 * i + (lane >> 4);
-      int rg = wrow0 + r;
-      if (rg > nrows - 1) rg = nrows - 1;
-      const int t = div_group(rg);
-      roff[i] = (uint32_t)((t - tok0) * a.qs_tok_bytes + (rg - t * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(r)) << 4));
-    }
-    const uint32_t st_a = lds0 + wave * kStageBytes, st_b = lds0 + kLdsRing + wave * kStageBytes;
-    const uint32_t frag = l32 * kRow + ((g ^ tile_swz(l32)) << 4);  // this lane's chunk 0 of row l32; ^ (s << 5), + 32 m rows
-#pragma unroll
-    for (int i = 0; i < 16; ++i) lds_direct_load16(qb, roff[i], st_a + i * 4 * kRow);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) lds_direct_load16(dob, roff[i], st_b + i * 4 * kRow);
-    wait_vm<16>();  // lse and Q are here
-    elemx8 qt[2][8], ot[2][8];
-#pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int s = 0; s < 8; ++s) qt[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(st_a + 32 * m * kRow + (frag ^ (s << 5))));
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the place is filled again
-#pragma unroll
-    for (int i = 0; i < 16; ++i) lds_direct_load16(ob, roff[i], st_a + i * 4 * kRow);
-    wait_vm<16>();  // dO is here
-#pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int s = 0; s < 8; ++s) dof[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(st_b + 32 * m * kRow + (frag ^ (s << 5))));
-    wait_vm<0>();  // O is here
-#pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int s = 0; s < 8; ++s) ot[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(st_a + 32 * m * kRow + (frag ^ (s << 5))));
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // nothing of this wave still reads where tile 0 will land
-    fence();
-#pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      float part = 0.f;
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        qf[m][s] = to_acc_regs(qt[m][s]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)ot[m][s][i];
-      }
-      delta[m] = pair_sum(part);  // this lane's half of d, then the sum of the lane pair
-      lse2[m] = valid[m] ? lse_row[m] * kLog2e : INFINITY;  // rows past the task: P = exp2(-inf) = 0
-    }
-  }
-  // -delta of the lane's row in all 16 registers of a vector: the C operand of a tile's first dP MFMA, so that
-  // dS = P * (what the MFMAs leave) costs one instruction per element
-  f32x16 ndl[2];
-#pragma unroll
-  for (int m = 0; m < 2; ++m)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) ndl[m][r] = -delta[m];
-  int wrow1 = wrow0 + 63;
-  if (wrow1 > nrows - 1) wrow1 = nrows - 1;
-  const bool wave_live = wrow0 < nrows;
-  int lim_first = 0x7fffffff, lim_last = -1;
-  if (wave_live) {
-    lim_first = a.causal ? wrow0 / G + shift : lk - 1;
-    if (lim_first > lk - 1) lim_first = lk - 1;
-    lim_last = a.causal ? wrow1 / G + shift : lk - 1;
-    if (lim_last > lk - 1) lim_last = lk - 1;
-  }
-
   // ---- K/V tile fetch: this wave brings rows 8 w .. 8 w + 7 of the K tile and of the V tile, four rows per
   // instruction.  Tiles that lie wholly inside the prefix take a form without per-lane address arithmetic (a scalar
   // base that advances by one tile, per-lane offsets that never change); rows past the prefix read the zero row.
@@ -318,6 +214,113 @@ next_block:
     }
   };
 
+  // The first two tiles are requested before the block's own rows: they land in the ring while the rows pass through
+  // the part of LDS behind it.
+  if (ntiles > 0) {
+    issue_tile(0, 0);
+    issue_tile(1, 1);
+  }
+
+  // ---- this lane's two rows: Q and dO as B operands (row l32 of a sub-block, d = 16 s + 8 g .. +7), statistics
+  int row[2], tok[2], lim[2];
+  bool valid[2];
+  float lse2[2], delta[2];
+  accop_t qf[2][8];
+  elemx8 dof[2][8];
+  // The wave's 64 rows of Q, dO and O come through LDS: LDS-direct loads bring four whole rows of 256 bytes per
+  // instruction, and the lanes then read their operand fragments (row l32 of a sub-block, chunk 2 s + g) from there.
+  // Loaded straight into the operand layout, every load instruction touched 32 rows, 32 bytes of each, and the address
+  // unit takes about a cycle per cache line it has to look up: 48 such loads per wave took 7.7 us to *issue*, a third
+  // of what a block of a 1024-token document then spent in its tile loop.  The rows use the 24 KB per wave that lie
+  // behind the tile ring (the 32 rows of a sub-block of Q, dO and O at a time), so the ring is free for the first tiles
+  // meanwhile, and each wave reads only what it has loaded itself: no barrier.
+  // Before that, and also in one batch, the lse of the lane's two rows (the opaque statements that move Q into the
+  // accumulation registers order memory accesses around themselves: no load may be left between them).
+  float lse_row[2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    row[m] = row_wg + (wave * 2 + m) * 32 + l32;
+    valid[m] = row[m] < nrows;
+    // A row past the task (the last block of a task only) reads the task's last row instead, without a branch: with
+    // lse2 = +inf its P and dS are zero whatever Q and dO hold, as long as they are finite, and nothing of it is stored.
+    const int rc = valid[m] ? row[m] : nrows - 1;
+    tok[m] = div_group(rc);
+    const int hg = rc - tok[m] * G;
+    int lm = a.causal ? tok[m] + shift : lk - 1;
+    if (lm > lk - 1) lm = lk - 1;
+    lim[m] = lm;
+    lse_row[m] = a.lse_tok ? reinterpret_cast<const float *>(a.lse_tok + qs_task + (int64_t)tok[m] * a.qs_tok_bytes)[kvh * G + hg]
+                           : a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]];
+  }
+  const int wrow0 = row_wg + wave * 64;
+  {
+    // offsets from the block's first token: instruction i brings rows 4 i + lane / 16 of the wave, lane % 16 the
+    // position of the 16-byte chunk in the (swizzled) LDS row
+    const int tok0 = div_group(row_wg);
+    const int64_t blk = qs_task + (int64_t)tok0 * a.qs_tok_bytes + (int64_t)kvh * G * kHeadDim * 2;
+    const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + blk, *dob = reinterpret_cast<const uint8_t *>(a.dout) + blk,
+                  *ob = reinterpret_cast<const uint8_t *>(a.out) + blk;
+    uint32_t roff[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = 4 * i + (lane >> 4);
+      int rg = wrow0 + r;
+      if (rg > nrows - 1) rg = nrows - 1;
+      const int t = div_group(rg);
+      roff[i] = (uint32_t)((t - tok0) * a.qs_tok_bytes + (rg - t * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(r)) << 4));
+    }
+    const uint32_t stg = lds0 + kLdsRing + wave * kRowsLds;  // [Q | dO | O] of one sub-block, 8 KB each
+    const uint32_t frag = l32 * kRow + ((g ^ tile_swz(l32)) << 4);  // this lane's chunk 0 of row l32; ^ (s << 5)
+    elemx8 qt[2][8], ot[2][8];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lds_direct_load16(qb, roff[8 * m + i], stg + i * 4 * kRow);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lds_direct_load16(dob, roff[8 * m + i], stg + kTile + i * 4 * kRow);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) lds_direct_load16(ob, roff[8 * m + i], stg + 2 * kTile + i * 4 * kRow);
+      wait_vm<0>();  // (the first tiles, requested before, and lse as well)
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        qt[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(stg + (frag ^ (s << 5))));
+        dof[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(stg + kTile + (frag ^ (s << 5))));
+        ot[m][s] = *static_cast<const DISTCA_LDS elemx8 *>(lds_ptr(stg + 2 * kTile + (frag ^ (s << 5))));
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the place is filled again
+    }
+    fence();
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      float part = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        qf[m][s] = to_acc_regs(qt[m][s]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part += (float)dof[m][s][i] * (float)ot[m][s][i];
+      }
+      delta[m] = pair_sum(part);  // this lane's half of d, then the sum of the lane pair
+      lse2[m] = valid[m] ? lse_row[m] * kLog2e : INFINITY;  // rows past the task: P = exp2(-inf) = 0
+    }
+  }
+  // -delta of the lane's row in all 16 registers of a vector: the C operand of a tile's first dP MFMA, so that
+  // dS = P * (what the MFMAs leave) costs one instruction per element
+  f32x16 ndl[2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ndl[m][r] = -delta[m];
+  int wrow1 = wrow0 + 63;
+  if (wrow1 > nrows - 1) wrow1 = nrows - 1;
+  const bool wave_live = wrow0 < nrows;
+  int lim_first = 0x7fffffff, lim_last = -1;
+  if (wave_live) {
+    lim_first = a.causal ? wrow0 / G + shift : lk - 1;
+    if (lim_first > lk - 1) lim_first = lk - 1;
+    lim_last = a.causal ? wrow1 / G + shift : lk - 1;
+    if (lim_last > lk - 1) lim_last = lk - 1;
+  }
+
   f32x16 dqacc[2][4];
 #pragma unroll
   for (int m = 0; m < 2; ++m)
@@ -343,12 +346,6 @@ next_block:
     asm volatile("" : "+v"(k_ad[i]), "+v"(t_ad[i]));
   }
 
-  wait_vm<0>();  // the counted waits below cover the tile loads only
-  __syncthreads();  // every wave has read the rows it staged in the ring's stages, which the tiles may now fill
-  if (ntiles > 0) {
-    issue_tile(0, 0);
-    issue_tile(1, 1);
-  }
 
   // One tile.  MASKED: the tile straddles the diagonal or the end of the prefix, compare and select per element.
   auto tile = [&](auto stage, int key0, auto masked) __attribute__((always_inline)) {  // stage: an int or a constant
@@ -517,7 +514,7 @@ next_block:
     }
   }
   {
-    const uint32_t out_b = lds0 + kLdsRing + wave * kStageBytes;
+    const uint32_t out_b = lds0 + kLdsRing + wave * kRowsLds;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
