@@ -117,6 +117,7 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   // (a jump back rather than a loop statement: without MERGE the body below is then straight-line code, exactly the
   // kernel that takes one block per item)
   int mblk = mb_first;
+  bool requested = false;  // MERGE: the first sub-block's rows of this block are already on their way
 next_block:
   // MERGE: the thread index is made opaque once per block, so that what derives from it is computed afresh for every
   // block instead of being carried, and partly spilled, across the whole body
@@ -253,33 +254,38 @@ next_block:
                            : a.lse[(int64_t)(kvh * G + hg) * a.total_q + q0 + tok[m]];
   }
   const int wrow0 = row_wg + wave * 64;
-  {
-    // offsets from the block's first token: instruction i brings rows 4 i + lane / 16 of the wave, lane % 16 the
-    // position of the 16-byte chunk in the (swizzled) LDS row
-    const int tok0 = div_group(row_wg);
-    const int64_t blk = qs_task + (int64_t)tok0 * a.qs_tok_bytes + (int64_t)kvh * G * kHeadDim * 2;
-    const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + blk, *dob = reinterpret_cast<const uint8_t *>(a.dout) + blk,
-                  *ob = reinterpret_cast<const uint8_t *>(a.out) + blk;
-    uint32_t roff[16];
+  const uint32_t stg = lds0 + kLdsRing + wave * kRowsLds;  // [Q | dO | O] of one sub-block, 8 KB each
+  // requests sub-block m of the wave's rows in block `blk` of the task: instruction i brings rows 32 m + 4 i + lane / 16
+  // of the wave, lane % 16 being the position of the 16-byte chunk in the (swizzled) LDS row
+  auto request_rows = [&](int blk, int m) {
+    const int rw = blk * kRowsWg;
+    const int tok0 = div_group(rw);
+    const int64_t base = qs_task + (int64_t)tok0 * a.qs_tok_bytes + (int64_t)kvh * G * kHeadDim * 2;
+    const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q) + base, *dob = reinterpret_cast<const uint8_t *>(a.dout) + base,
+                  *ob = reinterpret_cast<const uint8_t *>(a.out) + base;
+    uint32_t roff[8];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int r = 4 * i + (lane >> 4);
-      int rg = wrow0 + r;
+    for (int i = 0; i < 8; ++i) {
+      const int r = 32 * m + 4 * i + (lane >> 4);
+      int rg = rw + wave * 64 + r;
       if (rg > nrows - 1) rg = nrows - 1;
       const int t = div_group(rg);
       roff[i] = (uint32_t)((t - tok0) * a.qs_tok_bytes + (rg - t * G) * (kHeadDim * 2) + (((lane & 15) ^ tile_swz(r)) << 4));
     }
-    const uint32_t stg = lds0 + kLdsRing + wave * kRowsLds;  // [Q | dO | O] of one sub-block, 8 KB each
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_direct_load16(qb, roff[i], stg + i * 4 * kRow);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_direct_load16(dob, roff[i], stg + kTile + i * 4 * kRow);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_direct_load16(ob, roff[i], stg + 2 * kTile + i * 4 * kRow);
+  };
+  {
     const uint32_t frag = l32 * kRow + ((g ^ tile_swz(l32)) << 4);  // this lane's chunk 0 of row l32; ^ (s << 5)
     elemx8 qt[2][8], ot[2][8];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) lds_direct_load16(qb, roff[8 * m + i], stg + i * 4 * kRow);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) lds_direct_load16(dob, roff[8 * m + i], stg + kTile + i * 4 * kRow);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) lds_direct_load16(ob, roff[8 * m + i], stg + 2 * kTile + i * 4 * kRow);
+      // MERGE: the first sub-block's rows were requested before the previous block of the item stored its results
+      if (!(MERGE && m == 0 && requested)) request_rows(mblk, m);
       wait_vm<0>();  // (the first tiles, requested before, and lse as well)
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
@@ -499,6 +505,15 @@ next_block:
   for (; p < ntiles; ++p) advance(p);
   wait_vm<0>();  // nothing may still be on its way into LDS when the workgroup ends
 
+  // MERGE: the next block's first rows are requested now and arrive while this block's results are stored; the dQ rows
+  // then leave through the wave's stage of the ring, which every wave has left (the barrier), instead of through the
+  // rows' place.
+  if constexpr (MERGE) {
+    requested = mblk + 1 < mb_end;
+    __syncthreads();
+    if (requested) request_rows(mblk + 1, 0);
+  }
+
   // ---- epilogue: the row statistics for the dK/dV kernel, which runs after this one (stored here rather than where
   // they are made: the wait that precedes the tile loop would have to see the stores through as well), and the dQ rows.
   // A lane holds half of each of its two rows in pieces of 8 bytes (registers 4*cq..+3 of block db hold d0..d0+3):
@@ -514,7 +529,7 @@ next_block:
     }
   }
   {
-    const uint32_t out_b = lds0 + kLdsRing + wave * kRowsLds;
+    const uint32_t out_b = MERGE ? lds0 + wave * kStageBytes : stg;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
