@@ -46,7 +46,10 @@ constexpr int kVOff = kStatOff + kStages * kStatBytes;
 // Of the eight 16-element slices over d of a wave's V rows, the first kVRegSlices* stay in registers as B operands
 // beside K (as many as fit without spills inside the block loops: 12 fewer of a block's 72 LDS reads, -2 %); the
 // rest is read from LDS every block.
-constexpr int kVRegSlicesOwn = 6;     // the (task, key block) form
+#ifndef DISTCA_VREG_OWN
+#define DISTCA_VREG_OWN 6
+#endif
+constexpr int kVRegSlicesOwn = DISTCA_VREG_OWN;  // the (task, key block) form
 #ifndef DISTCA_VREG_SHARED
 #define DISTCA_VREG_SHARED 4
 #endif

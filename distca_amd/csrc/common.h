@@ -80,6 +80,15 @@ __device__ __forceinline__ float pair_sum(float x) { return x + __shfl_xor(x, 32
 // barrier before any wave reads the destination.  M0 is written here and used by nothing
 // else in these kernels.
 __device__ __forceinline__ uint32_t uniform32(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+// A pointer that is the same in every lane, moved to scalar registers.  Where the compiler cannot prove that (the value
+// derives from a work item read through LDS), it keeps a vector copy, and under pressure parks that copy in scratch
+// memory: the reload's wait then also waits for every LDS-direct load in flight, which it does not count as its own.
+template <typename T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+  const uint64_t u = reinterpret_cast<uint64_t>(p);
+  const uint64_t hi = uniform32((uint32_t)(u >> 32)), lo = uniform32((uint32_t)u);
+  return reinterpret_cast<T *>((hi << 32) | lo);
+}
 __device__ __forceinline__ void lds_direct_load16(const void *gbase, uint32_t voff, uint32_t lds_base) {
   const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
   const uint64_t gbu = ((uint64_t)uniform32((uint32_t)(gb >> 32)) << 32) | uniform32((uint32_t)gb);
