@@ -84,7 +84,9 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   const int nitems = a.sched[0];
   int item, kvh;
   if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
-  const int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  int4 it4 = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  it4.x = uniform_int(it4.x);
+  it4.y = uniform_int(it4.y);
   const int task = it4.x;
 
   // The task's bounds and offsets: every load is issued before the first is used (the optional arrays are read
@@ -94,9 +96,11 @@ __global__ __launch_bounds__(kThreads, 1) void ca_bwd_dq64_kernel(BwdArgs a) {
   const int32_t *kvp = a.kv_off ? a.kv_off + task : ck;
   const int64_t *spare = reinterpret_cast<const int64_t *>(a.zero_row);
   const int64_t *qsp = a.qs_task_off ? a.qs_task_off + task : spare, *dqp = a.dq_task_off ? a.dq_task_off + task : spare;
-  const int q0 = cq[0], q1 = cq[1], k0 = ck[0], k1 = ck[1], ks = *kvp;
-  const int64_t qs_given = *qsp, dq_given = *dqp;
+  const int q0_ = cq[0], q1_ = cq[1], k0_ = ck[0], k1_ = ck[1], ks_ = *kvp;
+  const int64_t qs_given_ = *qsp, dq_given_ = *dqp;
   fence();
+  const int q0 = uniform_int(q0_), q1 = uniform_int(q1_), k0 = uniform_int(k0_), k1 = uniform_int(k1_), ks = uniform_int(ks_);
+  const int64_t qs_given = uniform_int64(qs_given_), dq_given = uniform_int64(dq_given_);
   const int64_t qs_task = a.qs_task_off ? qs_given : (int64_t)q0 * a.qs_tok_bytes;
   const int64_t dq_task = a.dq_task_off ? dq_given : (int64_t)q0 * a.dq_tok_bytes;
   const int lq = q1 - q0;

@@ -80,6 +80,15 @@ __device__ __forceinline__ float pair_sum(float x) { return x + __shfl_xor(x, 32
 // barrier before any wave reads the destination.  M0 is written here and used by nothing
 // else in these kernels.
 __device__ __forceinline__ uint32_t uniform32(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+// Values that are the same in every lane, moved to scalar registers: what is loaded from memory counts as differing
+// from lane to lane for the compiler, and so does everything computed from it (a task's bounds, its base pointers,
+// loop limits), which then costs vector instructions and registers where scalar ones would do.
+__device__ __forceinline__ int uniform_int(int x) { return (int)uniform32((uint32_t)x); }
+__device__ __forceinline__ int64_t uniform_int64(int64_t x) {
+  const uint64_t u = (uint64_t)x;
+  const uint64_t hi = uniform32((uint32_t)(u >> 32)), lo = uniform32((uint32_t)u);  // (each half widened as unsigned)
+  return (int64_t)((hi << 32) | lo);
+}
 // A pointer that is the same in every lane, moved to scalar registers.  Where the compiler cannot prove that (the value
 // derives from a work item read through LDS), it keeps a vector copy, and under pressure parks that copy in scratch
 // memory: the reload's wait then also waits for every LDS-direct load in flight, which it does not count as its own.
