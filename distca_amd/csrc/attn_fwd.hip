@@ -72,13 +72,17 @@ __global__ __launch_bounds__(kFwdWaves * 64, (MSUB == 1 && kFwdWaves == 4 ? 2 : 
   const int nitems = a.sched[0];
   int item, kvh;
   if (!take_item(a.tickets, nitems, a.hkv, reinterpret_cast<int32_t *>(lds), item, kvh)) return;
-  const int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  // (the item's fields and the task's bounds are moved to scalar registers as they are read: what derives from them,
+  // base pointers, loop limits and tile addresses, is then scalar arithmetic)
+  int4 it = reinterpret_cast<const int4 *>(a.sched + a.sched_items_off)[item];
+  it.x = uniform_int(it.x);
+  it.y = uniform_int(it.y);
   const int task = it.x;
 
-  const int q0 = a.cu_q[task];
-  const int lq = a.cu_q[task + 1] - q0;
-  const int lk = a.cu_k[task + 1] - a.cu_k[task];
-  const int ks = a.kv_off ? a.kv_off[task] : a.cu_k[task];
+  const int q0 = uniform_int(a.cu_q[task]);
+  const int lq = uniform_int(a.cu_q[task + 1]) - q0;
+  const int lk = uniform_int(a.cu_k[task + 1]) - uniform_int(a.cu_k[task]);
+  const int ks = uniform_int(a.kv_off ? a.kv_off[task] : a.cu_k[task]);
   const int G = a.group;
   const int shift = lk - lq;
 
@@ -118,8 +122,8 @@ next_block:
   const int ntiles = nvis > 0 ? (nvis + kFwdKV - 1) / kFwdKV : 0;
 
   // ---- per-lane rows
-  const uint8_t *qbytes = reinterpret_cast<const uint8_t *>(a.q) + (a.q_task_off ? a.q_task_off[task] : (int64_t)q0 * a.q_tok_bytes);
-  uint8_t *obytes = reinterpret_cast<uint8_t *>(a.out) + (a.out_task_off ? a.out_task_off[task] : (int64_t)q0 * a.out_tok_bytes);
+  const uint8_t *qbytes = reinterpret_cast<const uint8_t *>(a.q) + uniform_int64(a.q_task_off ? a.q_task_off[task] : (int64_t)q0 * a.q_tok_bytes);
+  uint8_t *obytes = reinterpret_cast<uint8_t *>(a.out) + uniform_int64(a.out_task_off ? a.out_task_off[task] : (int64_t)q0 * a.out_tok_bytes);
   int row[MSUB], tok[MSUB], lim[MSUB];
   bool valid[MSUB];
   const elem_t *qptr[MSUB];
