@@ -35,7 +35,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch on the default 131072-token workload: rocprofv3 --pmc FETCH_SIZE (x2.000) and
 # WRITE_SIZE (x1.000), factors from the pack kernels' known copy sizes in the same run
-MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.95e9, "ca_bwd_dkdv64_kernel": 22.58e9, "ca_bwd_dq64_kernel": 13.34e9}
+MEASURED_TRAFFIC_BYTES = {"ca_fwd_kernel": 10.95e9, "ca_bwd_dkdv64_kernel": 22.69e9, "ca_bwd_dq64_kernel": 13.24e9}
 
 
 def log(*a):
