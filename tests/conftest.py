@@ -22,7 +22,7 @@ def cuda():
 
 def pytest_sessionfinish(session, exitstatus):
     """Writes the raw error figures of every attention comparison of this run (tests/helpers.py: PARITY_LOG) to
-    gpurun_out/parity_errors.json, worst case per (test function, tensor): the asserted figures are measured
+    parity_errors.json in the run's output folder, worst case per (test function, tensor): the asserted figures are measured
     above the bf16 rounding floor, and this file is where the raw ones can be audited."""
     try:
         import json
