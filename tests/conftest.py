@@ -26,9 +26,10 @@ def pytest_sessionfinish(session, exitstatus):
     above the bf16 rounding floor, and this file is where the raw ones can be audited."""
     try:
         import json
+        import torch
         import helpers
-        if not helpers.PARITY_LOG:
-            return
+        if not helpers.PARITY_LOG or not torch.cuda.is_available():
+            return   # (a session without a GPU only holds the helper's own tests: it must not replace a GPU run's report)
         worst = {}
         for test_id, what, e in helpers.PARITY_LOG:
             name = test_id.split("::")[-1].split("[")[0]
